@@ -1,0 +1,397 @@
+"""CPU oracle for the XAttention prefill path.  TEST INFRASTRUCTURE ONLY.
+
+This module is a checker, not a product path: only ``tests/``, the smoke test
+and the ``cpu_baseline`` leg of the benchmark may import it.  The shipped
+operator never calls into it and raises when its HIP library is missing.
+
+It restates, in plain device-agnostic torch, the algorithm of the reference
+(``mit-han-lab/x-attention``); every function names the reference lines it
+follows (paths relative to the reference checkout):
+
+* :func:`antidiagonal_scores`      - xattn/src/Xattention.py:84-94 + 182-185
+                                     (== xattn/src/kernels.py:219-230)
+* :func:`estimate_chunk_block_sums`- xattn/src/Xattention.py:174-252 (torch branch)
+* :func:`find_blocks_chunked`      - xattn/src/utils.py:44-191 (prefill branch)
+* :func:`xattn_estimate`           - xattn/src/Xattention.py:13-299
+* :func:`default_chunk_size`       - xattn/src/Xattention.py:322-331
+* :func:`block_sparse_attention`   - the un-vendored ``block_sparse_attn==0.0.1``
+                                     call at xattn/src/Xattention.py:377-391,
+                                     restated as dense softmax attention under
+                                     the expanded block mask (and token-causal).
+* :func:`Xattention_prefill`       - xattn/src/Xattention.py:302-402
+
+Pinning status (what independent evidence each function is checked against,
+see tests/test_oracle_*.py):
+
+* antidiagonal_scores: brute force over the full Q.K^T on tiny inputs
+  (sum of S x S antidiagonals), and pointer-form vs concatenation-form.
+* estimate_chunk_block_sums: torch.softmax in fp64 on the brute-force scores,
+  row-mass invariant (a real q-block row sums to block_size/stride), zeros
+  above the block diagonal, zero padded rows, chunk-size independence when
+  ``pad0_quirk=False``.
+* find_blocks_chunked: golden input/output vectors produced by the
+  reference's own ``xattn/src/utils.py`` (tests/golden/find_blocks_*.pt,
+  made by tests/golden/make_find_blocks_golden.py), plus a brute-force
+  sorted-prefix enumeration.
+* block_sparse_attention: PARITY UNPINNED against block_sparse_attn itself
+  (third-party CUDA, absent from the reference tree, no reference test holds
+  results for it).  It is pinned to the mathematics only: all-True mask ==
+  torch scaled_dot_product_attention, and a per-row python loop on tiny
+  inputs.
+* xattn_estimate / Xattention_prefill glue: invariants (block-tril, forced
+  sink/diagonal, keep_sink row, keep_recent diagonal) and tiny hand cases.
+"""
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+NEG_INF = float("-inf")
+
+
+# --------------------------------------------------------------------------- #
+# A3: antidiagonal (stride-S reversed reshape) scores
+# --------------------------------------------------------------------------- #
+def reshape_inverse(query_states, key_states, stride):
+    """Concatenation form of the stride-S reshape, select_mode="inverse", kdb=1.
+
+    Follows xattn/src/Xattention.py:84-94: keys take token ``n*S+i`` into
+    feature slab ``i``; queries take token ``m*S+(S-1-i)`` into slab ``i``.
+    """
+    rk = torch.cat([key_states[:, :, i::stride, :] for i in range(stride)], dim=-1)
+    rq = torch.cat(
+        [query_states[:, :, (stride - 1 - i) :: stride, :] for i in range(stride)],
+        dim=-1,
+    )
+    return rq, rk
+
+
+def antidiagonal_scores(query_states, key_states, stride):
+    """score[m, n] = sum_i Q[m*S + S-1-i] . K[n*S + i]  (un-scaled).
+
+    xattn/src/Xattention.py:182-185 applied to :func:`reshape_inverse`;
+    identical to the pointer arithmetic of xattn/src/kernels.py:219-230.
+    """
+    rq, rk = reshape_inverse(query_states, key_states, stride)
+    return torch.matmul(rq, rk.transpose(2, 3))
+
+
+# --------------------------------------------------------------------------- #
+# A5: threshold block selection
+# --------------------------------------------------------------------------- #
+def find_blocks_chunked(
+    input_tensor,
+    current_index,
+    threshold,
+    num_to_choose,
+    decoding,
+    mode="both",
+    causal=True,
+):
+    """Per q-block row, keep blocks until their mass reaches ``threshold``.
+
+    Restates the prefill branch of xattn/src/utils.py:87-191 including its
+    incidental behaviours: fp64 arithmetic (:87), per-head tensor thresholds
+    (:91-95), forced sink and diagonal columns (:99-106), the
+    ``[0, forced_sum, others...]`` prefix that is one slot longer than the
+    forced set when sink and diagonal coincide (:115-124), rewriting of the
+    unselected ranks to column 0 before the scatter (:142, :164) and the
+    clearing of columns past the chunk's last diagonal (:176-180).
+    """
+    assert threshold is None or num_to_choose is None
+    if threshold is None:
+        raise NotImplementedError("selection by block count is not implemented upstream")
+    bsz, heads, rows, cols = input_tensor.shape
+    if mode == "prefill" and decoding:
+        return torch.ones_like(input_tensor, dtype=torch.bool)
+    if mode == "decode" and not decoding:
+        raise NotImplementedError("decode-mode masks are outside the prefill path")
+    dev = input_tensor.device
+    x = input_tensor.to(torch.float64)
+
+    total = x.sum(dim=-1, keepdim=True)
+    if isinstance(threshold, torch.Tensor):
+        tau = threshold.to(torch.float64).to(dev)
+        required = total * tau.reshape(1, -1, 1, 1).expand(bsz, heads, rows, 1)
+    else:
+        required = total * threshold
+
+    def scatter_rows(mask, index):
+        flat_mask = mask.view(bsz, heads * rows, cols)
+        flat_index = index.view(bsz, heads * rows, cols)
+        row_id = torch.arange(heads * rows, device=dev).unsqueeze(-1)
+        flat_mask[:, row_id, flat_index] = True
+        return flat_mask.view(bsz, heads, rows, cols)
+
+    zero_col = torch.zeros((bsz, heads, rows, 1), dtype=torch.float64, device=dev)
+    if causal:
+        forced = torch.zeros_like(x, dtype=torch.bool)
+        forced[..., 0] = True
+        eye = torch.eye(rows, dtype=torch.bool, device=dev)
+        forced[..., current_index : current_index + rows] = eye
+        others_sorted, _ = torch.sort(x.masked_fill(forced, 0), dim=-1, descending=True)
+        forced_sum = torch.where(forced, x, 0.0).sum(dim=-1, keepdim=True)
+        ranked_values = torch.cat([zero_col, forced_sum, others_sorted[..., :-2]], dim=-1)
+        _, order = torch.sort(
+            torch.where(forced, 100000 * (1 + x), x), dim=-1, descending=True
+        )
+        mass_before = torch.cat([zero_col, ranked_values[..., :-1]], dim=-1).cumsum(dim=-1)
+        keep = mass_before < required
+        mask = scatter_rows(forced.clone(), torch.where(keep, order, 0))
+        # columns after the last diagonal of this chunk never survive (:176-180)
+        mask[..., current_index + rows :] = False
+    else:
+        values_sorted, order = torch.sort(x, dim=-1, descending=True)
+        mass_before = torch.cat([zero_col, values_sorted[..., :-1]], dim=-1).cumsum(dim=-1)
+        keep = mass_before < required
+        mask = scatter_rows(
+            torch.zeros_like(x, dtype=torch.bool), torch.where(keep, order, 0)
+        )
+    return mask
+
+
+# --------------------------------------------------------------------------- #
+# A2 / A4: per-chunk softmax + block sums (torch branch), and the estimate
+# --------------------------------------------------------------------------- #
+def estimate_chunk_block_sums(
+    reshaped_query,
+    reshaped_key,
+    chunk_idx,
+    *,
+    head_dim,
+    stride,
+    norm,
+    block_size,
+    chunk_size,
+    k_chunk_num,
+    q_chunk_num,
+    k_reshaped_num_to_pad,
+    q_reshaped_num_to_pad,
+    causal,
+    pad0_quirk,
+    out_dtype,
+):
+    """Block sums of softmax(antidiagonal scores) for one query chunk.
+
+    Follows xattn/src/Xattention.py:174-252.  ``pad0_quirk=True`` keeps the
+    literal behaviour of line 201: with no key padding the slice
+    ``[..., -0:]`` covers every column, so each query chunk sees only the
+    keys of its own chunk.  ``pad0_quirk=False`` skips that line when there is
+    no padding, which is what the reference's Triton branch computes
+    (xattn/src/kernels.py:42-66 sweeps from key column 0).
+    """
+    bsz, heads = reshaped_query.shape[:2]
+    rcs = chunk_size // stride
+    rbs = block_size // stride
+    offset_chunks = k_chunk_num - q_chunk_num
+    cq = reshaped_query[:, :, chunk_idx * rcs : (chunk_idx + 1) * rcs, :]
+    w = torch.matmul(cq, reshaped_key.transpose(2, 3))
+    w = w / math.sqrt(head_dim) / stride / norm
+    last_padded = chunk_idx == q_chunk_num - 1 and q_reshaped_num_to_pad != 0
+    if causal:
+        cm = torch.zeros((bsz, heads, rcs, rcs * k_chunk_num), device=w.device)
+        if k_reshaped_num_to_pad > 0 or pad0_quirk:
+            cm[..., (-k_reshaped_num_to_pad):] = NEG_INF
+        c0 = (chunk_idx + offset_chunks) * rcs
+        c1 = c0 + rcs
+        cm[..., c0:c1] = torch.triu(
+            torch.full((rcs, rcs), NEG_INF, device=w.device), diagonal=1
+        )
+        if last_padded:
+            cm[:, :, (-q_reshaped_num_to_pad):, :] = NEG_INF
+        cm[..., c1:] = NEG_INF
+        w = w + cm
+    w = F.softmax(w, dim=-1, dtype=torch.float32).to(out_dtype)
+    if last_padded:
+        w[:, :, (-q_reshaped_num_to_pad):, :] = 0
+    sums = w.view(bsz, heads, rcs // rbs, rbs, -1, rbs).sum(dim=-1).sum(dim=-2)
+    return sums
+
+
+def xattn_estimate(
+    query_states,
+    key_states,
+    block_size,
+    stride,
+    norm=1,
+    softmax=True,
+    threshold=0.9,
+    chunk_size=16384,
+    select_mode="inverse",
+    use_triton=False,
+    causal=True,
+    kdb=1,
+    keep_sink=False,
+    keep_recent=False,
+    pad0_quirk=True,
+):
+    """(attn_sums, simple_masks), both ``[B, H, Nq_blocks_padded, Nk_blocks_padded]``.
+
+    Restates xattn/src/Xattention.py:13-299 for ``select_mode="inverse"``,
+    ``kdb=1``, ``softmax=True`` on whatever device the inputs live on.
+    ``use_triton`` is accepted for signature parity and ignored; the only
+    semantic difference between the two upstream branches that survives in
+    exact arithmetic is ``pad0_quirk`` (see :func:`estimate_chunk_block_sums`).
+    """
+    if select_mode not in ("inverse", "") or kdb != 1 or not softmax:
+        raise NotImplementedError("only select_mode='inverse', kdb=1, softmax=True")
+    bsz, kv_heads, k_len, head_dim = key_states.shape
+    _, heads, q_len, _ = query_states.shape
+    assert heads == kv_heads
+
+    k_pad = -k_len % chunk_size
+    q_pad = -q_len % chunk_size
+    k_chunk_num = (k_len + k_pad) // chunk_size
+    q_chunk_num = (q_len + q_pad) // chunk_size
+    k_block_num = (k_len + k_pad) // block_size
+    q_block_num = (q_len + q_pad) // block_size
+    assert k_chunk_num >= q_chunk_num
+    pk = F.pad(key_states, (0, 0, 0, k_pad), value=0) if k_pad else key_states
+    pq = F.pad(query_states, (0, 0, 0, q_pad), value=0) if q_pad else query_states
+    rq, rk = reshape_inverse(pq, pk, stride)
+    blocks_per_chunk = chunk_size // block_size
+
+    sums, masks = [], []
+    for c in range(q_chunk_num):
+        s = estimate_chunk_block_sums(
+            rq,
+            rk,
+            c,
+            head_dim=head_dim,
+            stride=stride,
+            norm=norm,
+            block_size=block_size,
+            chunk_size=chunk_size,
+            k_chunk_num=k_chunk_num,
+            q_chunk_num=q_chunk_num,
+            k_reshaped_num_to_pad=k_pad // stride,
+            q_reshaped_num_to_pad=q_pad // stride,
+            causal=causal,
+            pad0_quirk=pad0_quirk,
+            out_dtype=pq.dtype,
+        )
+        m = find_blocks_chunked(
+            s,
+            k_block_num - q_block_num + c * blocks_per_chunk,
+            threshold,
+            None,
+            decoding=False,
+            mode="prefill",
+            causal=causal,
+        )
+        sums.append(s)
+        masks.append(m)
+    attn_sums = torch.cat(sums, dim=-2)
+    simple_masks = torch.cat(masks, dim=-2)
+
+    if causal:
+        tril = torch.tril(
+            torch.ones(q_block_num, q_block_num, dtype=torch.bool, device=simple_masks.device)
+        )
+        tail = simple_masks[:, :, -q_block_num:, -q_block_num:]
+        simple_masks[:, :, -q_block_num:, -q_block_num:] = tail & tril
+    if keep_sink:
+        simple_masks[:, :, 0, :] = True
+    if keep_recent:
+        eye = torch.eye(q_block_num, dtype=torch.bool, device=simple_masks.device)
+        tail = simple_masks[:, :, -q_block_num:, -q_block_num:]
+        simple_masks[:, :, -q_block_num:, -q_block_num:] = tail | eye
+    return attn_sums, simple_masks
+
+
+def default_chunk_size(k_len):
+    """Operator's default chunk rule, xattn/src/Xattention.py:322-331."""
+    p = 1 << (k_len - 1).bit_length()
+    return int(max(min(max(2048, p), 128 * 1024 * 2048 // p), 2048))
+
+
+# --------------------------------------------------------------------------- #
+# A6: block-sparse attention as dense masked softmax attention
+# --------------------------------------------------------------------------- #
+def block_sparse_attention(
+    query_states,
+    key_states,
+    value_states,
+    block_mask,
+    causal=True,
+    block_size=128,
+    softmax_scale=None,
+    row_tile=1024,
+):
+    """softmax(Q K^T * scale + M) V in fp32, M = block mask expanded x block_size
+    and (when ``causal``) the bottom-right-aligned token-causal mask.
+
+    ``block_mask`` is ``[B, H, ceil(Lq/bs), ceil(Lk/bs)]`` bool.  K/V may carry
+    fewer heads than Q (grouped-query attention); query head h reads KV head
+    ``h // (H / H_kv)``.  A query row with no visible key yields zeros.
+    Output is ``[B, H, Lq, d]`` in the input dtype.
+    """
+    bsz, heads, q_len, d = query_states.shape
+    kv_heads, k_len = key_states.shape[1], key_states.shape[2]
+    group = heads // kv_heads
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(d)
+    kf = key_states.float().repeat_interleave(group, dim=1)
+    vf = value_states.float().repeat_interleave(group, dim=1)
+    out = torch.empty((bsz, heads, q_len, d), dtype=torch.float32, device=query_states.device)
+    kpos = torch.arange(k_len, device=query_states.device)
+    for r0 in range(0, q_len, row_tile):
+        r1 = min(q_len, r0 + row_tile)
+        qpos = torch.arange(r0, r1, device=query_states.device)
+        s = torch.matmul(query_states[:, :, r0:r1].float(), kf.transpose(2, 3)) * scale
+        allow = block_mask[:, :, qpos // block_size][:, :, :, kpos // block_size]
+        if causal:
+            allow = allow & (kpos[None, :] <= qpos[:, None] + (k_len - q_len))
+        s = s.masked_fill(~allow, NEG_INF)
+        p = torch.softmax(s, dim=-1)
+        p = torch.nan_to_num(p, nan=0.0)
+        out[:, :, r0:r1] = torch.matmul(p, vf)
+    return out.to(query_states.dtype)
+
+
+def Xattention_prefill(
+    query_states,
+    key_states,
+    value_states,
+    stride,
+    norm=1,
+    threshold=0.8,
+    block_size=128,
+    use_triton=False,
+    causal=True,
+    kdb=1,
+    chunk_size=None,
+    keep_sink=False,
+    keep_recent=False,
+    pad0_quirk=True,
+    return_mask=False,
+):
+    """Estimate -> block mask -> masked attention, xattn/src/Xattention.py:302-402."""
+    bsz, heads, k_len, d = key_states.shape
+    q_len = query_states.shape[2]
+    assert block_size == 128 and bsz == 1
+    q_block_num = (q_len + block_size - 1) // block_size
+    k_block_num = (k_len + block_size - 1) // block_size
+    if chunk_size is None:
+        chunk_size = default_chunk_size(k_len)
+    _, mask = xattn_estimate(
+        query_states,
+        key_states,
+        block_size=block_size,
+        stride=stride,
+        norm=norm,
+        threshold=threshold,
+        select_mode="inverse",
+        use_triton=use_triton,
+        causal=causal,
+        chunk_size=chunk_size,
+        kdb=kdb,
+        keep_sink=keep_sink,
+        keep_recent=keep_recent,
+        pad0_quirk=pad0_quirk,
+    )
+    mask = mask[:, :, :q_block_num, :k_block_num].contiguous()
+    out = block_sparse_attention(
+        query_states, key_states, value_states, mask, causal=causal, block_size=block_size
+    )
+    return (out, mask) if return_mask else out

@@ -1,0 +1,130 @@
+"""Pins oracle.find_blocks_chunked: golden vectors from the reference's own
+xattn/src/utils.py (tests/golden/find_blocks_golden.pt), an independent
+brute-force enumeration, and selection properties."""
+import os
+
+import pytest
+import torch
+
+from oracle import xattn_oracle as O
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "find_blocks_golden.pt")
+
+
+def load_cases():
+    return torch.load(GOLD, weights_only=True)
+
+
+def test_golden_vectors_from_reference():
+    cases = load_cases()
+    assert len(cases) >= 20
+    for c in cases:
+        tau = c["threshold"] if c["threshold_is_tensor"] else float(c["threshold"])
+        got = O.find_blocks_chunked(
+            c["x"].clone(), c["current_index"], tau, None, decoding=False, mode="prefill", causal=c["causal"]
+        )
+        assert got.dtype == torch.bool
+        assert torch.equal(got, c["mask"]), c["name"]
+
+
+def brute_select_row(vals, tau, causal, diag, limit):
+    """Sorted-prefix enumeration for one row, written from the rule rather than
+    the tensor program: forced = {0, diag}; visit the rest by descending value
+    and keep a block while the mass gathered before it is below tau*total."""
+    n = len(vals)
+    total = sum(vals)
+    need = total * tau
+    keep = [False] * n
+    if causal:
+        forced = sorted({0, diag})
+        mass = 0.0
+        for f in forced:
+            keep[f] = True
+            mass += vals[f]
+        rest = sorted((i for i in range(n) if i not in forced), key=lambda i: -vals[i])
+        extra = 1 if len(forced) == 1 else 0  # one-slot-longer prefix, utils.py:115-124
+        gathered = []
+        for rank, i in enumerate(rest):
+            before = 0.0 if rank < extra else mass + sum(gathered[: rank - extra])
+            if before < need:
+                keep[i] = True
+            gathered.append(vals[i])
+        for i in range(limit, n):
+            keep[i] = False
+    else:
+        order = sorted(range(n), key=lambda i: -vals[i])
+        mass = 0.0
+        dropped = False
+        for i in order:
+            if mass < need:
+                keep[i] = True
+            else:
+                dropped = True
+            mass += vals[i]
+        if dropped:
+            keep[0] = True  # unselected ranks are scattered to column 0, utils.py:164
+    return keep
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("tau", [0.0, 0.5, 0.9, 1.0])
+def test_bruteforce_enumeration(causal, tau):
+    g = torch.Generator().manual_seed(int(tau * 100) + causal)
+    rows, cols, cur = 6, 14, 8 if causal else 0
+    x = torch.rand(1, 2, rows, cols, generator=g, dtype=torch.float64) + 0.01
+    if causal:
+        for r in range(rows):
+            x[:, :, r, cur + r + 1 :] = 0
+    got = O.find_blocks_chunked(x, cur, tau, None, decoding=False, mode="prefill", causal=causal)
+    for h in range(2):
+        for r in range(rows):
+            vals = x[0, h, r].tolist()
+            want = brute_select_row(vals, tau, causal, cur + r, cur + rows)
+            if causal and tau == 1.0:
+                # zero-valued future blocks tie; compare only the causal part
+                want, have = want[: cur + r + 1], got[0, h, r, : cur + r + 1].tolist()
+            else:
+                have = got[0, h, r].tolist()
+            assert have == want, (h, r)
+
+
+def test_selection_properties():
+    g = torch.Generator().manual_seed(7)
+    rows, cols, cur = 8, 16, 8
+    x = torch.rand(1, 4, rows, cols, generator=g, dtype=torch.float64) ** 2 + 1e-3
+    for r in range(rows):
+        x[:, :, r, cur + r + 1 :] = 0
+    prev = None
+    for tau in (0.0, 0.2, 0.5, 0.8, 0.95):
+        m = O.find_blocks_chunked(x, cur, tau, None, decoding=False, mode="prefill", causal=True)
+        # forced sink + diagonal
+        assert m[..., 0].all()
+        assert all(m[0, :, r, cur + r].all() for r in range(rows))
+        # reaches the required mass
+        got = torch.where(m, x, 0.0).sum(-1)
+        assert (got >= tau * x.sum(-1) - 1e-12).all()
+        # minimality: dropping the smallest selected non-forced block falls below
+        for h in range(4):
+            for r in range(rows):
+                sel = [c for c in range(cols) if m[0, h, r, c] and c not in (0, cur + r)]
+                if sel:
+                    smallest = min(sel, key=lambda c: x[0, h, r, c].item())
+                    assert got[0, h, r] - x[0, h, r, smallest] < tau * x[0, h, r].sum()
+        # monotone in tau
+        if prev is not None:
+            assert (m | ~prev).all()
+        prev = m
+    m0 = O.find_blocks_chunked(x, cur, 0.0, None, decoding=False, mode="prefill", causal=True)
+    assert m0.sum().item() == 4 * rows * 2  # tau=0 -> forced blocks only
+
+
+def test_per_head_threshold_broadcast():
+    g = torch.Generator().manual_seed(9)
+    x = torch.rand(1, 3, 4, 12, generator=g, dtype=torch.float64)
+    taus = torch.tensor([0.2, 0.7, 0.95], dtype=torch.float32)
+    m = O.find_blocks_chunked(x, 0, taus, None, decoding=False, mode="prefill", causal=False)
+    for h in range(3):
+        mh = O.find_blocks_chunked(
+            x[:, h : h + 1], 0, float(taus[h].double()), None, decoding=False, mode="prefill", causal=False
+        )
+        assert torch.equal(m[:, h : h + 1], mh)
