@@ -1,0 +1,141 @@
+/* C ABI of libxattn_hip.so: the gfx950 (MI355X) kernels behind the XAttention
+ * prefill operator.
+ *
+ * Conventions shared by every entry point
+ *  - all pointers are DEVICE pointers unless a parameter says "host";
+ *  - q/k/v/out are bf16, laid out [head][token][128] with the feature dimension
+ *    contiguous; head and token strides are given in ELEMENTS and must be
+ *    multiples of 8 (16-byte rows), base pointers 16-byte aligned;
+ *  - batch is 1 (the reference asserts it, xattn/src/Xattention.py:357);
+ *  - K/V may carry fewer heads than Q: query head h reads KV head
+ *    h / (num_heads / num_kv_heads);
+ *  - `stream` is a hipStream_t passed as void*; work is enqueued on it and the
+ *    call returns without synchronising; nothing is allocated inside;
+ *  - the return value is XATTN_OK or a negative XATTN_ERR_* code; arguments are
+ *    validated on the host before anything is launched, nothing is thrown.
+ *
+ * Paths cited as xattn/... are files of mit-han-lab/x-attention.
+ */
+#ifndef XATTN_HIP_H
+#define XATTN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  XATTN_OK = 0,
+  XATTN_ERR_NULL = -1,      /* a required pointer is null                       */
+  XATTN_ERR_HEAD_DIM = -2,  /* head_dim != 128                                  */
+  XATTN_ERR_HEADS = -3,     /* num_heads not a positive multiple of kv heads    */
+  XATTN_ERR_SHAPE = -4,     /* lengths / block counts / pitches out of range    */
+  XATTN_ERR_ALIGN = -5,     /* pointer or stride not 16-byte aligned            */
+  XATTN_ERR_STRIDE = -6,    /* antidiagonal stride not one of 4, 8, 16          */
+  XATTN_ERR_WORKSPACE = -7, /* workspace too small                              */
+  XATTN_ERR_LAUNCH = -8     /* the HIP runtime refused the launch               */
+};
+
+/* Library ABI version (bumped when a signature changes). */
+int xattn_abi_version(void);
+
+/* Text for an XATTN_ERR_* code (static storage, never null). */
+const char* xattn_error_string(int code);
+
+/* ---------------------------------------------------------------------------
+ * Antidiagonal estimator.  Replaces, fused and without materialising the
+ * strided score matrix, the pair
+ *   flat_group_gemm_fuse_reshape   xattn/src/kernels.py:325-363 (kernel 197-235)
+ *   softmax_fuse_block_sum         xattn/src/kernels.py:238-289 (kernels 5-156)
+ * as driven by the chunk loop of xattn_estimate, xattn/src/Xattention.py:138-172
+ * (torch branch 174-252).
+ *
+ * Q and K are treated as zero-padded to multiples of chunk_size
+ * (Xattention.py:33-51).  With n_rq = q_len_padded/stride reshaped query rows
+ * and n_rk = k_len_padded/stride reshaped keys,
+ *   score[m][n] = sum_i Q[m*stride + stride-1-i] . K[n*stride + i]
+ * is scaled by `scale` (= 1/sqrt(128)/stride/norm), soft-maxed over the
+ * visible n of each row, and summed into (block_size/stride)^2 tiles:
+ *   block_sums[h][i][j], i < q_len_padded/block_size, j < k_len_padded/block_size.
+ * causal != 0: reshaped key n is visible to row m iff
+ *   k_lo(m) <= n <= m + (n_rk - n_rq)            (inclusive, Xattention.py:204-214)
+ * with k_lo = 0 when own_chunk_only == 0 (the reference's Triton branch) or the
+ * first reshaped key of the row's own chunk when own_chunk_only != 0 (what the
+ * reference's torch branch computes when k_len is a multiple of chunk_size,
+ * Xattention.py:201).  causal == 0: every n is visible, zero-padded keys
+ * included.  Rows m >= n_rq - (q_len_padded - q_len)/stride are all-zero
+ * (Xattention.py:237-238).
+ * Only query chunks [chunk_begin, chunk_end) are processed (rows of block_sums
+ * outside them are left untouched), so a caller may pipeline chunks on streams.
+ * `scores_out`, when non-null, receives the un-scaled scores of those chunks as
+ * fp32 [num_heads][n_rq][n_rk] (entries of tiles with no visible pair are left
+ * untouched) - the flat_group_gemm_fuse_reshape seam, for tests.
+ * `workspace` must hold xattn_estimate_workspace_bytes(...) bytes, where
+ * chunks_per_call is the largest chunk_end - chunk_begin used (<= 0: all chunks);
+ * the function returns 0 for arguments the estimator rejects.
+ */
+size_t xattn_estimate_workspace_bytes(int num_heads, int q_len, int k_len, int stride, int block_size,
+                                      int chunk_size, int chunks_per_call);
+
+int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, void* workspace,
+                              size_t workspace_bytes, float* scores_out, int num_heads,
+                              int num_kv_heads, int q_len, int k_len, int head_dim, int64_t q_stride_h,
+                              int64_t q_stride_n, int64_t k_stride_h, int64_t k_stride_n, int stride,
+                              int block_size, int chunk_size, int chunk_begin, int chunk_end, int causal,
+                              int own_chunk_only, float scale, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Threshold block selection.  Replaces find_blocks_chunked,
+ * xattn/src/utils.py:44-191 (prefill branch), together with the mask
+ * post-processing of xattn_estimate, xattn/src/Xattention.py:275-297.
+ *
+ * For q-block rows [row_begin, row_end) of every head: in fp64, required =
+ * tau[h] * sum(row).  causal != 0: column 0 and the diagonal column
+ * row + diag_offset are always kept; the remaining columns are visited by
+ * descending block sum and kept while (forced mass + mass of those visited
+ * before) < required; columns beyond the diagonal are cleared.  causal == 0:
+ * all columns are visited by descending block sum and kept while the mass
+ * visited before is < required; if any column is left out, column 0 is kept
+ * (utils.py:164).  keep_sink sets q-block row 0 entirely (Xattention.py:286-287);
+ * keep_recent sets the diagonal (288-297).  Ties in block sum are broken by
+ * ascending column.
+ * Outputs: mask [H][nq_blocks][nk_blocks] bytes (0/1);
+ *          col_idx [H][nq_blocks][idx_pitch] ascending kept columns that are
+ *          < list_cols and, when causal, hold a key visible to the row's last
+ *          query token given kv_off_tokens = k_len - q_len;  col_cnt [H][nq_blocks].
+ * col_idx/col_cnt may both be null.  nk_blocks <= 16384.
+ */
+int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uint8_t* mask,
+                        int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int num_heads,
+                        int nq_blocks, int nk_blocks, int row_begin, int row_end, int diag_offset,
+                        int causal, int keep_sink, int keep_recent, int list_cols, int q_len,
+                        int kv_off_tokens, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Block-sparse FlashAttention forward.  Replaces the call
+ *   block_sparse_attn_func(q, k, v, cu_q, cu_k, head_mask_type, None, mask,
+ *                          q_len, k_len, p_dropout=0, deterministic=True,
+ *                          is_causal=causal)      xattn/src/Xattention.py:377-391
+ * for one sequence (cu_seqlens = [0, len]) and per-head masks.  Query block
+ * qb (128 tokens) of head h visits the col_cnt[h][qb] key blocks listed in
+ * col_idx[h][qb][*] (arrays of idx_rows >= ceil(q_len/128) rows per head, each
+ * idx_pitch entries long, as xattn_select_blocks writes them); inside a block, when causal, key c is visible to query t
+ * iff c <= t + (k_len - q_len).  A query row with no visible key yields zeros.
+ * col_idx == col_cnt == null visits every visible block: dense FlashAttention,
+ * the baseline the speedup is quoted against.
+ */
+int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* out,
+                           const int32_t* col_idx, const int32_t* col_cnt, int64_t idx_pitch,
+                           int idx_rows, int num_heads, int num_kv_heads, int q_len, int k_len,
+                           int head_dim,
+                           int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
+                           int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
+                           int64_t o_stride_h, int64_t o_stride_n, int causal, float softmax_scale,
+                           void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XATTN_HIP_H */

@@ -1,0 +1,403 @@
+// Antidiagonal block-score estimator for gfx950.
+//
+// Fuses what the reference does with two Triton kernels and an HBM round trip
+// of the strided score matrix (flat_group_gemm_fuse_reshape,
+// xattn/src/kernels.py:197-235, then softmax_fuse_block_sum, :5-156; driven by
+// xattn/src/Xattention.py:138-172):
+//
+//  kernel 1 (estimate_gemm_kernel): a bf16 MFMA GEMM over the reshaped
+//    operands, gathered on the fly - reshaped key n at depth slab i is token
+//    n*S+i, reshaped query m is token m*S+S-1-i - with a 256x256 tile per
+//    workgroup and 128x128 per wavefront.  Scores are produced transposed
+//    (keys along accumulator rows) so one lane owns one query row.  In the
+//    epilogue each wavefront scales, masks, takes the row maximum over ITS 128
+//    keys, exponentiates against that local maximum and adds up groups of
+//    block_size/S keys.  It writes, per (query row, 128-key tile), the local
+//    maximum and sum, and per (query row, key block) the partial sum - 1/S of
+//    the score matrix, in fp32 - never the scores themselves.
+//  kernel 2 (estimate_normalize_kernel): per query row, combines the tile
+//    maxima/sums into the row's softmax statistics, rescales the partial sums
+//    and adds the block_size/S rows of each query block.
+#include "xattn_common.h"
+#include "xattn_hip.h"
+
+namespace xattn {
+
+constexpr int kTile = 256;       // workgroup tile edge (reshaped rows / keys)
+constexpr int kSub = 128;        // wavefront tile edge
+constexpr int kDepth = 64;       // bf16 per k-step (one 128-byte line per row)
+constexpr int kStageBytes = 2 * kTile * kDepth * 2;  // K' + Q' slabs of one stage
+
+struct EstParams {
+  const __bf16* q;
+  const __bf16* k;
+  int64_t q_sh, q_sn, k_sh, k_sn;
+  float* P;        // [H][nkb][rows]  partial block sums relative to the tile maximum
+  float* Mt;       // [H][nT][rows]   tile maximum (exp2 domain)
+  float* Lt;       // [H][nT][rows]   tile sum
+  float* scores;   // optional [H][n_rq][n_rk] raw scores
+  float* sums;     // [H][nqb][nkb] output block sums
+  int H, Hkv, Lq, Lk, S, rbs;
+  int n_rq, n_rk, nkb, nqb, nT;
+  int rcs;                  // reshaped rows per chunk
+  int row_begin, row_end;   // reshaped query rows handled by this call
+  int rows;                 // row_end - row_begin (pitch of P / Mt / Lt)
+  int off;                  // n_rk - n_rq: position of query row 0 on the key axis
+  int real_rows;            // query rows >= real_rows are padding
+  int causal, own_chunk_only;
+  float scale_log2;
+};
+
+// first / last visible reshaped key of reshaped query row m
+__device__ __forceinline__ int row_lo(const EstParams& p, int m) {
+  return (p.causal && p.own_chunk_only) ? (m / p.rcs) * p.rcs + p.off : 0;
+}
+__device__ __forceinline__ int row_hi(const EstParams& p, int m) {
+  return p.causal ? m + p.off : p.n_rk - 1;
+}
+
+// One k-step slab: 256 rows x 64 bf16 per operand.  8 lanes fetch one row's
+// 128-byte line; tokens past the real length read as zeros (the padding of
+// xattn/src/Xattention.py:33-51).
+__device__ __forceinline__ void load_slab(const __bf16* base, int64_t sn, int len, int first_row, int S,
+                                          int tok_in_group, int feat0, int tid, u32x4 (&st)[8]) {
+  const int c = tid & 7, r0 = tid >> 3;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int64_t tok = (int64_t)(first_row + r0 + 32 * it) * S + tok_in_group;
+    const bool ok = tok < len;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    u32x4 x = z;
+    if (ok) x = *reinterpret_cast<const u32x4*>(base + tok * sn + feat0 + c * 8);
+    st[it] = x;
+  }
+}
+
+// LDS slab layout: row r at byte r*128, its 16-byte chunk c stored at chunk
+// c ^ (r & 7) so that 8 lanes reading the same logical chunk of 8 consecutive
+// rows touch all banks.
+__device__ __forceinline__ void store_slab(char* slab, int tid, const u32x4 (&st)[8]) {
+  const int c = tid & 7, r0 = tid >> 3;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int r = r0 + 32 * it;
+    *reinterpret_cast<u32x4*>(slab + r * 128 + ((c ^ (r & 7)) << 4)) = st[it];
+  }
+}
+
+__device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk) {
+  return *reinterpret_cast<const bf16x8*>(slab + row * 128 + ((chunk ^ (row & 7)) << 4));
+}
+
+template <int RBS>
+__global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, hh = lane >> 5;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int head = blockIdx.z;
+  const int m0 = p.row_begin + blockIdx.y * kTile;
+  const int n0 = blockIdx.x * kTile;
+
+  // tiles without a visible (row, key) pair do nothing
+  {
+    const int m_last = (m0 + kTile - 1 < p.row_end ? m0 + kTile - 1 : p.row_end - 1);
+    if (n0 > row_hi(p, m_last)) return;
+    if (n0 + kTile - 1 < row_lo(p, m0)) return;
+  }
+
+  const int kvh = head / (p.H / p.Hkv);
+  const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
+  const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+
+  f32x16 acc[4][4];   // [key tile nt][query tile mt]
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+  const int steps = p.S * 2;
+  u32x4 stK[8], stQ[8];
+  load_slab(kbase, p.k_sn, p.Lk, n0, p.S, 0, 0, tid, stK);
+  load_slab(qbase, p.q_sn, p.Lq, m0, p.S, p.S - 1, 0, tid, stQ);
+  store_slab(lds, tid, stK);
+  store_slab(lds + kTile * 128, tid, stQ);
+  __syncthreads();
+
+  for (int t = 0; t < steps; ++t) {
+    char* cur = lds + (t & 1) * kStageBytes;
+    char* nxt = lds + ((t + 1) & 1) * kStageBytes;
+    const bool more = t + 1 < steps;
+    if (more) {
+      const int i = (t + 1) >> 1, f0 = ((t + 1) & 1) * kDepth;
+      load_slab(kbase, p.k_sn, p.Lk, n0, p.S, i, f0, tid, stK);
+      load_slab(qbase, p.q_sn, p.Lq, m0, p.S, p.S - 1 - i, f0, tid, stQ);
+    }
+    const char* slabK = cur;
+    const char* slabQ = cur + kTile * 128;
+#pragma unroll
+    for (int ss = 0; ss < 4; ++ss) {
+      bf16x8 fa[4], fb[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        fa[x] = read_frag(slabK, wn * kSub + x * 32 + r, ss * 2 + hh);
+        fb[x] = read_frag(slabQ, wm * kSub + x * 32 + r, ss * 2 + hh);
+      }
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma32(fa[nt], fb[mt], acc[nt][mt]);
+    }
+    if (more) {
+      store_slab(nxt, tid, stK);
+      store_slab(nxt + kTile * 128, tid, stQ);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: this wavefront's 128 keys x 128 query rows
+  const int nbase = n0 + wn * kSub;       // first key of the wavefront tile
+  const int T = nbase / kSub;
+  if (nbase >= p.n_rk) return;
+  float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
+  float* Mst = p.Mt + ((int64_t)head * p.nT + T) * p.rows;
+  float* Lst = p.Lt + ((int64_t)head * p.nT + T) * p.rows;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int m = m0 + wm * kSub + mt * 32 + r;
+    const bool row_ok = m < p.row_end;
+    const int lo = row_lo(p, m), hi = row_hi(p, m);
+    if (p.scores && row_ok) {
+      float* dst = p.scores + ((int64_t)head * p.n_rq + m) * p.n_rk;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int n = nbase + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
+          if (n < p.n_rk) dst[n] = acc[nt][mt][v];
+        }
+    }
+    float x[4][16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int n = nbase + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
+        const bool vis = n >= lo && n <= hi && n < p.n_rk;
+        x[nt][v] = vis ? acc[nt][mt][v] * p.scale_log2 : -INFINITY;
+        mx = fmaxf(mx, x[nt][v]);
+      }
+    mx = fmaxf(mx, swap_half(mx));
+    const float safe = (mx == -INFINITY) ? 0.f : mx;
+    float tot = 0.f;
+    const int mrel = m - p.row_begin;
+    constexpr int G = RBS / 8;   // 8-key groups (one per accumulator quad pair) per key block
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      float part[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float s = 0.f;
+#pragma unroll
+        for (int t2 = 0; t2 < 4; ++t2) s += fast_exp2(x[nt][g * 4 + t2] - safe);
+        part[g] = s + swap_half(s);
+        tot += part[g];
+      }
+      // part[g] covers keys nbase + nt*32 + 8g .. +7
+      if (G == 1) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int kb = (nbase + nt * 32 + g * 8) / RBS;
+          if (row_ok && kb < p.nkb && hh == (g & 1)) Pst[(int64_t)kb * p.rows + mrel] = part[g];
+        }
+      } else if (G == 2) {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const int kb = (nbase + nt * 32 + g * 16) / RBS;
+          if (row_ok && kb < p.nkb && hh == g) Pst[(int64_t)kb * p.rows + mrel] = part[2 * g] + part[2 * g + 1];
+        }
+      } else {
+        const int kb = (nbase + nt * 32) / RBS;
+        if (row_ok && kb < p.nkb && hh == 0)
+          Pst[(int64_t)kb * p.rows + mrel] = part[0] + part[1] + part[2] + part[3];
+      }
+    }
+    if (row_ok && hh == 0) {
+      Mst[mrel] = mx;
+      Lst[mrel] = tot;
+    }
+  }
+}
+
+// One workgroup = 64 consecutive reshaped query rows (lane <-> row) of one
+// head; its 4 wavefronts split the key range.
+template <int RBS>
+__global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
+  __shared__ float redM[4][64];
+  __shared__ float redL[4][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int head = blockIdx.y;
+  const int m = p.row_begin + blockIdx.x * 64 + lane;
+  const bool row_ok = m < p.row_end;
+  const int mc = row_ok ? m : p.row_end - 1;
+  const int mrel = mc - p.row_begin;
+  const int lo = row_lo(p, mc);
+  int hi = row_hi(p, mc);
+  hi = hi < p.n_rk - 1 ? hi : p.n_rk - 1;
+  const float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
+  const float* Mst = p.Mt + (int64_t)head * p.nT * p.rows;
+  const float* Lst = p.Lt + (int64_t)head * p.nT * p.rows;
+
+  // pass 1: row statistics from the per-tile maxima and sums
+  float M = -INFINITY, L = 0.f;
+  const int T_lo = lo / kSub, T_hi = hi / kSub;
+  for (int T = T_lo + wave; T <= T_hi; T += 4) {
+    const float mt = Mst[(int64_t)T * p.rows + mrel];
+    const float lt = Lst[(int64_t)T * p.rows + mrel];
+    const float Mn = fmaxf(M, mt);
+    const float safe = (Mn == -INFINITY) ? 0.f : Mn;
+    L = L * fast_exp2(M - safe) + lt * fast_exp2(mt - safe);
+    M = Mn;
+  }
+  redM[wave][lane] = M;
+  redL[wave][lane] = L;
+  __syncthreads();
+  float Mr = fmaxf(fmaxf(redM[0][lane], redM[1][lane]), fmaxf(redM[2][lane], redM[3][lane]));
+  const float safe = (Mr == -INFINITY) ? 0.f : Mr;
+  float Lr = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) Lr += redL[w][lane] * fast_exp2(redM[w][lane] - safe);
+  const bool real = row_ok && mc < p.real_rows && Lr > 0.f;
+  const float inv = real ? 1.f / Lr : 0.f;
+
+  // pass 2: rescale each key block's partial sum and add the RBS rows of a query block
+  const int kb_lo = lo / RBS, kb_hi = hi / RBS;
+  float* out = p.sums + ((int64_t)head * p.nqb + mc / RBS) * p.nkb;
+  for (int kb = wave; kb < p.nkb; kb += 4) {
+    float w = 0.f;
+    if (real && kb >= kb_lo && kb <= kb_hi) {
+      const int T = (kb * RBS) / kSub;
+      w = Pst[(int64_t)kb * p.rows + mrel] * fast_exp2(Mst[(int64_t)T * p.rows + mrel] - safe) * inv;
+    }
+#pragma unroll
+    for (int d = 1; d < RBS; d <<= 1) w += __shfl_xor(w, d, 64);
+    if (row_ok && (lane % RBS) == 0) out[kb] = w;
+  }
+}
+
+}  // namespace xattn
+
+using namespace xattn;
+
+namespace {
+struct Geometry {
+  int q_pad, k_pad, n_rq, n_rk, nqb, nkb, nT, rcs, q_chunks;
+};
+
+bool geometry(int q_len, int k_len, int stride, int block_size, int chunk_size, Geometry* g) {
+  if (q_len <= 0 || k_len <= 0 || chunk_size <= 0) return false;
+  if (chunk_size % block_size) return false;
+  const int64_t qp = ((int64_t)q_len + chunk_size - 1) / chunk_size * chunk_size;
+  const int64_t kp = ((int64_t)k_len + chunk_size - 1) / chunk_size * chunk_size;
+  if (kp > (int64_t)1 << 30 || kp < qp) return false;
+  g->q_pad = (int)(qp - q_len);
+  g->k_pad = (int)(kp - k_len);
+  g->n_rq = (int)(qp / stride);
+  g->n_rk = (int)(kp / stride);
+  g->nqb = (int)(qp / block_size);
+  g->nkb = (int)(kp / block_size);
+  g->nT = (g->n_rk + kSub - 1) / kSub;
+  g->rcs = chunk_size / stride;
+  g->q_chunks = (int)(qp / chunk_size);
+  return true;
+}
+
+size_t workspace_bytes(int H, const Geometry& g, int rows) {
+  return (size_t)H * rows * ((size_t)g.nkb + 2 * (size_t)g.nT) * sizeof(float);
+}
+}  // namespace
+
+extern "C" size_t xattn_estimate_workspace_bytes(int num_heads, int q_len, int k_len, int stride,
+                                                 int block_size, int chunk_size, int chunks_per_call) {
+  Geometry g;
+  if (num_heads <= 0 || block_size != 128 || (stride != 4 && stride != 8 && stride != 16)) return 0;
+  if (!geometry(q_len, k_len, stride, block_size, chunk_size, &g)) return 0;
+  int c = (chunks_per_call <= 0 || chunks_per_call > g.q_chunks) ? g.q_chunks : chunks_per_call;
+  return workspace_bytes(num_heads, g, c * g.rcs);
+}
+
+extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, void* workspace,
+                                         size_t workspace_size, float* scores_out, int num_heads,
+                                         int num_kv_heads, int q_len, int k_len, int head_dim,
+                                         int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
+                                         int64_t k_stride_n, int stride, int block_size, int chunk_size,
+                                         int chunk_begin, int chunk_end, int causal, int own_chunk_only,
+                                         float scale, void* stream) {
+  if (!q || !k || !block_sums || !workspace) return XATTN_ERR_NULL;
+  if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
+  if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
+  if (block_size != 128 || (stride != 4 && stride != 8 && stride != 16)) return XATTN_ERR_STRIDE;
+  Geometry g;
+  if (!geometry(q_len, k_len, stride, block_size, chunk_size, &g)) return XATTN_ERR_SHAPE;
+  if (chunk_begin < 0 || chunk_end > g.q_chunks || chunk_begin >= chunk_end) return XATTN_ERR_SHAPE;
+  if (q_stride_h % 8 || q_stride_n % 8 || k_stride_h % 8 || k_stride_n % 8) return XATTN_ERR_ALIGN;
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) return XATTN_ERR_ALIGN;
+
+  EstParams p;
+  p.q = static_cast<const __bf16*>(q);
+  p.k = static_cast<const __bf16*>(k);
+  p.q_sh = q_stride_h; p.q_sn = q_stride_n; p.k_sh = k_stride_h; p.k_sn = k_stride_n;
+  p.H = num_heads; p.Hkv = num_kv_heads; p.Lq = q_len; p.Lk = k_len; p.S = stride;
+  p.rbs = block_size / stride;
+  p.n_rq = g.n_rq; p.n_rk = g.n_rk; p.nkb = g.nkb; p.nqb = g.nqb; p.nT = g.nT; p.rcs = g.rcs;
+  p.row_begin = chunk_begin * g.rcs;
+  p.row_end = chunk_end * g.rcs;
+  p.rows = p.row_end - p.row_begin;
+  p.off = g.n_rk - g.n_rq;
+  p.real_rows = g.n_rq - g.q_pad / stride;
+  p.causal = causal ? 1 : 0;
+  p.own_chunk_only = own_chunk_only ? 1 : 0;
+  p.scale_log2 = scale * kLog2e;
+  p.scores = scores_out;
+  p.sums = block_sums;
+  if (workspace_size < workspace_bytes(num_heads, g, p.rows)) return XATTN_ERR_WORKSPACE;
+  float* ws = static_cast<float*>(workspace);
+  p.P = ws;
+  p.Mt = ws + (size_t)num_heads * g.nkb * p.rows;
+  p.Lt = p.Mt + (size_t)num_heads * g.nT * p.rows;
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid1((g.n_rk + kTile - 1) / kTile, (p.rows + kTile - 1) / kTile, num_heads);
+  const dim3 grid2((p.rows + 63) / 64, num_heads);
+  if (grid1.y > 65535 || grid1.z > 65535 || grid2.y > 65535) return XATTN_ERR_SHAPE;
+  const size_t lds = 2 * (size_t)kStageBytes;
+  hipError_t e = hipSuccess;
+  switch (p.rbs) {
+    case 8:
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&estimate_gemm_kernel<8>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return XATTN_ERR_LAUNCH;
+      hipLaunchKernelGGL(estimate_gemm_kernel<8>, grid1, dim3(256), lds, s, p);
+      hipLaunchKernelGGL(estimate_normalize_kernel<8>, grid2, dim3(256), 0, s, p);
+      break;
+    case 16:
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&estimate_gemm_kernel<16>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return XATTN_ERR_LAUNCH;
+      hipLaunchKernelGGL(estimate_gemm_kernel<16>, grid1, dim3(256), lds, s, p);
+      hipLaunchKernelGGL(estimate_normalize_kernel<16>, grid2, dim3(256), 0, s, p);
+      break;
+    default:
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&estimate_gemm_kernel<32>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return XATTN_ERR_LAUNCH;
+      hipLaunchKernelGGL(estimate_gemm_kernel<32>, grid1, dim3(256), lds, s, p);
+      hipLaunchKernelGGL(estimate_normalize_kernel<32>, grid2, dim3(256), 0, s, p);
+      break;
+  }
+  return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
+}

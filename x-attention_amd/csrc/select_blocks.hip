@@ -1,0 +1,188 @@
+// Threshold block selection for gfx950: one wavefront per (head, q-block row).
+//
+// Replaces find_blocks_chunked (xattn/src/utils.py:44-191, prefill branch) and
+// the mask post-processing of xattn_estimate (xattn/src/Xattention.py:275-297).
+// The reference runs ~15 eager torch ops over an fp64 copy of the block sums
+// (two full sorts, a cumsum, an advanced-index scatter) and synchronises the
+// device once per chunk; here a row's candidates are sorted by a bitonic
+// network in LDS (only the columns up to the diagonal when causal - a
+// "segmented" sort whose size follows the row), the fp64 prefix sum is a
+// wavefront scan, and the kernel emits the final mask row plus the compacted,
+// ascending column list the attention kernel walks.
+#include "xattn_common.h"
+#include "xattn_hip.h"
+
+namespace xattn {
+
+struct SelParams {
+  const float* sums;
+  const double* tau;
+  uint8_t* mask;
+  int32_t* col_idx;
+  int32_t* col_cnt;
+  int64_t idx_pitch;
+  int H, nqb, nkb, row_begin, row_end, diag_offset;
+  int causal, keep_sink, keep_recent, list_cols, q_len, kv_off;
+  int npow2;   // LDS key capacity (power of two >= nkb)
+};
+
+__device__ __forceinline__ double wave_sum(double x) {
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) x += __shfl_xor(x, d, 64);
+  return x;
+}
+
+__global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  uint64_t* keys = reinterpret_cast<uint64_t*>(smem);
+  uint8_t* flags = reinterpret_cast<uint8_t*>(smem + (size_t)p.npow2 * 8);
+
+  const int lane = threadIdx.x;
+  const int rows = p.row_end - p.row_begin;
+  const int head = blockIdx.x / rows;
+  const int row = p.row_begin + blockIdx.x % rows;
+  const float* x = p.sums + ((int64_t)head * p.nqb + row) * p.nkb;
+  const int diag = row + p.diag_offset;
+
+  // candidates: columns [0, ncand); when causal nothing beyond the diagonal can be kept
+  int ncand = p.nkb;
+  if (p.causal) ncand = diag + 1 < p.nkb ? diag + 1 : p.nkb;
+  if (ncand < 0) ncand = 0;
+  int np2 = 64;
+  while (np2 < ncand) np2 <<= 1;
+
+  double total = 0.0;
+  for (int c = lane; c < np2; c += 64) {
+    uint64_t key = 0;   // padding sorts last and carries an out-of-range column
+    if (c < ncand) {
+      const float v = x[c];
+      total += (double)v;
+      const bool forced = p.causal && (c == 0 || c == diag);
+      // block sums are >= 0, so their bit pattern orders like the value;
+      // low word = ~column makes equal sums come out by ascending column
+      const uint32_t bits = forced ? 0u : __float_as_uint(v > 0.f ? v : 0.f);
+      key = ((uint64_t)bits << 32) | (uint32_t)(~(uint32_t)c);
+    }
+    keys[c] = key;
+  }
+  for (int c = lane; c < p.nkb; c += 64) flags[c] = 0;
+  total = wave_sum(total);
+  const double required = total * p.tau[head];
+  double forced_sum = 0.0;
+  if (p.causal && ncand > 0) {
+    forced_sum = (double)x[0];
+    if (diag != 0 && diag < p.nkb) forced_sum += (double)x[diag];
+  }
+  __syncthreads();
+
+  // bitonic sort, descending
+  for (int k = 2; k <= np2; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = lane; t < (np2 >> 1); t += 64) {
+        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));
+        const int l = i | j;
+        const uint64_t a = keys[i], b = keys[l];
+        const bool up = (i & k) == 0;        // this pair's run is descending
+        if ((a < b) == up) {
+          keys[i] = b;
+          keys[l] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  // fp64 exclusive prefix over the sorted values; rank kept while mass before it < required
+  const int per = np2 >> 6;
+  double local = 0.0;
+  for (int u = 0; u < per; ++u) local += (double)__uint_as_float((uint32_t)(keys[lane * per + u] >> 32));
+  double incl = local;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const double o = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += o;
+  }
+  double before = forced_sum + (incl - local);
+  int dropped = 0;
+  for (int u = 0; u < per; ++u) {
+    const uint64_t key = keys[lane * per + u];
+    const uint32_t col = ~(uint32_t)key;
+    if (col < (uint32_t)ncand) {
+      const bool forced = p.causal && ((int)col == 0 || (int)col == diag);
+      if (before < required) flags[col] = 1;
+      else if (!forced) dropped = 1;
+    }
+    before += (double)__uint_as_float((uint32_t)(key >> 32));
+  }
+  const bool any_dropped = __any(dropped);
+  __syncthreads();
+  if (lane == 0) {
+    if (p.causal) {
+      if (p.nkb > 0) flags[0] = 1;
+      if (diag >= 0 && diag < p.nkb) flags[diag] = 1;
+    } else if (any_dropped) {
+      flags[0] = 1;     // unselected ranks scatter to column 0 (utils.py:164)
+    }
+    if (p.keep_recent && diag >= 0 && diag < p.nkb) flags[diag] = 1;
+  }
+  __syncthreads();
+  if (p.keep_sink && row == 0)
+    for (int c = lane; c < p.nkb; c += 64) flags[c] = 1;
+  __syncthreads();
+
+  uint8_t* mrow = p.mask + ((int64_t)head * p.nqb + row) * p.nkb;
+  for (int c = lane; c < p.nkb; c += 64) mrow[c] = flags[c];
+
+  if (p.col_idx) {
+    int32_t* list = p.col_idx + ((int64_t)head * p.nqb + row) * p.idx_pitch;
+    const int q_last = (row * 128 + 127 < p.q_len ? row * 128 + 127 : p.q_len - 1) + p.kv_off;
+    int count = 0;
+    for (int c0 = 0; c0 < p.nkb; c0 += 64) {
+      const int c = c0 + lane;
+      bool keep = c < p.nkb && flags[c] && c < p.list_cols;
+      if (p.causal) keep = keep && (c * 128 <= q_last);
+      const uint64_t ballot = __ballot(keep);
+      const int pos = count + __popcll(ballot & ((1ull << lane) - 1ull));
+      if (keep && pos < p.idx_pitch) list[pos] = c;
+      count += __popcll(ballot);
+    }
+    if (lane == 0) p.col_cnt[head * p.nqb + row] = count < p.idx_pitch ? count : (int)p.idx_pitch;
+  }
+}
+
+}  // namespace xattn
+
+using namespace xattn;
+
+extern "C" int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uint8_t* mask,
+                                   int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int num_heads,
+                                   int nq_blocks, int nk_blocks, int row_begin, int row_end,
+                                   int diag_offset, int causal, int keep_sink, int keep_recent,
+                                   int list_cols, int q_len, int kv_off_tokens, void* stream) {
+  if (!block_sums || !tau_per_head || !mask) return XATTN_ERR_NULL;
+  if ((col_idx == nullptr) != (col_cnt == nullptr)) return XATTN_ERR_NULL;
+  if (num_heads <= 0 || nq_blocks <= 0 || nk_blocks <= 0 || nk_blocks > 16384) return XATTN_ERR_SHAPE;
+  if (row_begin < 0 || row_end > nq_blocks || row_begin >= row_end) return XATTN_ERR_SHAPE;
+  if (col_idx && idx_pitch < 1) return XATTN_ERR_SHAPE;
+  if (diag_offset < 0) return XATTN_ERR_SHAPE;
+  SelParams p;
+  p.sums = block_sums; p.tau = tau_per_head; p.mask = mask; p.col_idx = col_idx; p.col_cnt = col_cnt;
+  p.idx_pitch = idx_pitch; p.H = num_heads; p.nqb = nq_blocks; p.nkb = nk_blocks;
+  p.row_begin = row_begin; p.row_end = row_end; p.diag_offset = diag_offset;
+  p.causal = causal ? 1 : 0; p.keep_sink = keep_sink ? 1 : 0; p.keep_recent = keep_recent ? 1 : 0;
+  p.list_cols = list_cols; p.q_len = q_len; p.kv_off = kv_off_tokens;
+  int np2 = 64;
+  while (np2 < nk_blocks) np2 <<= 1;
+  p.npow2 = np2;
+  const size_t lds = (size_t)np2 * 8 + (((size_t)nk_blocks + 15) & ~(size_t)15);
+  const int64_t grid = (int64_t)num_heads * (row_end - row_begin);
+  if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
+  if (lds > 48 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&select_blocks_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return XATTN_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(select_blocks_kernel, dim3((unsigned)grid), dim3(64), lds,
+                     static_cast<hipStream_t>(stream), p);
+  return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
+}

@@ -1,0 +1,39 @@
+// Shared device helpers for the gfx950 XAttention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace xattn {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+
+constexpr int kWave = 64;
+constexpr int kHeadDim = 128;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// D[32x32] += A[32x16] * B[16x32], bf16 in, fp32 accumulate.
+// Lane l (r = l % 32, h = l / 32) supplies A[r][8h..8h+7] and B[8h..8h+7][r];
+// it receives D[8*(v/4) + 4h + v%4][r] in element v of the accumulator.
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+  bf16x2 p;
+  p[0] = (__bf16)lo;
+  p[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, p);
+}
+
+// value held by the lane 32 positions away (the other half-wave)
+__device__ __forceinline__ float swap_half(float x) { return __shfl_xor(x, 32, 64); }
+
+}  // namespace xattn

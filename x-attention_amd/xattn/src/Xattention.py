@@ -1,0 +1,278 @@
+"""XAttention prefill operator on MI355X: same names, arguments and results as
+``xattn/src/Xattention.py`` of mit-han-lab/x-attention, computed by the HIP
+kernels of ``libxattn_hip.so``.
+
+Differences a caller can rely on:
+
+* ``key_states`` / ``value_states`` may carry fewer heads than ``query_states``
+  (grouped-query attention by KV-head sharing; the reference asserts equal
+  head counts and its callers ``repeat_kv`` first).  Passing repeated K/V
+  still works.
+* ``use_triton`` selects which of the reference's two estimator branches is
+  reproduced, both on the HIP kernels: ``True`` (the default everywhere in the
+  reference's integrations) gives the Triton-branch result, where every query
+  chunk sees all earlier keys; ``False`` gives the torch-branch result, which
+  for ``k_len % chunk_size == 0`` restricts each query chunk to the keys of
+  its own chunk (xattn/src/Xattention.py:201).
+* block sums are kept in fp32 for the selection; ``attn_sums`` is cast to the
+  query dtype only on return.
+* tensors must be bf16 on a ROCm device; there is no CPU or eager fallback.
+"""
+import math
+
+import torch
+
+from . import hip_backend as _hb
+
+__all__ = ["Xattention_prefill", "xattn_estimate", "default_chunk_size", "estimate_and_select", "block_sparse_attention"]
+
+BLOCK = 128
+
+
+def default_chunk_size(k_len):
+    """Chunk rule of xattn/src/Xattention.py:322-331 (chunk * 2^ceil(log2 k_len) <= 2^28)."""
+    p = 1 << (k_len - 1).bit_length()
+    return int(max(min(max(2048, p), 128 * 1024 * 2048 // p), 2048))
+
+
+def _stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _check_qk(x, name):
+    if not x.is_cuda:
+        raise _hb.XattnHipError(f"{name} must live on a ROCm device (no CPU fallback exists)")
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be torch.bfloat16, got {x.dtype}")
+    if x.dim() != 4 or x.shape[0] != 1:
+        raise AssertionError(f"{name} must be [1, heads, len, 128] (batch 1 only)")
+    if x.shape[-1] != 128:
+        raise AssertionError("head_dim must be 128")
+    if x.stride(-1) != 1 or x.stride(1) % 8 or x.stride(2) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    return x
+
+
+def _tau_per_head(threshold, heads, device):
+    """float, 0-d tensor or [H] tensor -> float64 [H] on device, rounded the way
+    the reference rounds it (a tensor keeps its own precision, utils.py:91-92)."""
+    if isinstance(threshold, torch.Tensor):
+        t = threshold.detach().to(torch.float64).reshape(-1)
+        if t.numel() == 1:
+            t = t.expand(heads)
+        if t.numel() != heads:
+            raise ValueError(f"threshold tensor must have 1 or {heads} entries")
+        return t.contiguous().to(device)
+    return torch.full((heads,), float(threshold), dtype=torch.float64, device=device)
+
+
+def estimate_and_select(
+    query_states,
+    key_states,
+    stride,
+    threshold,
+    chunk_size,
+    causal=True,
+    norm=1,
+    use_triton=True,
+    keep_sink=False,
+    keep_recent=False,
+    block_size=BLOCK,
+    want_lists=True,
+    dump_scores=False,
+):
+    """Runs the estimator and selection kernels.
+
+    Returns a dict with fp32 ``sums`` [H, Nq_p, Nk_p], uint8 ``mask`` of the same
+    shape, and (when ``want_lists``) ``col_idx`` [H, Nq_p, pitch] / ``col_cnt``
+    [H, Nq_p] for :func:`block_sparse_attention`.
+    """
+    lib = _hb.lib()
+    q = _check_qk(query_states, "query_states")
+    k = _check_qk(key_states, "key_states")
+    if k.device != q.device:
+        k = k.to(q.device)
+    heads, q_len = q.shape[1], q.shape[2]
+    kv_heads, k_len = k.shape[1], k.shape[2]
+    if block_size != BLOCK:
+        raise AssertionError("block_size must be 128")
+    if stride not in (4, 8, 16):
+        raise ValueError("stride must be 4, 8 or 16")
+    if heads % kv_heads:
+        raise AssertionError("query heads must be a multiple of key/value heads")
+    if chunk_size % block_size:
+        raise AssertionError("chunk_size must be a multiple of block_size")
+    dev = q.device
+    q_pad = -q_len % chunk_size
+    k_pad = -k_len % chunk_size
+    q_chunks = (q_len + q_pad) // chunk_size
+    k_chunks = (k_len + k_pad) // chunk_size
+    assert k_chunks >= q_chunks
+    nqb, nkb = (q_len + q_pad) // block_size, (k_len + k_pad) // block_size
+    own_chunk_only = bool(causal) and (not use_triton) and k_pad == 0
+
+    with torch.cuda.device(dev):
+        stream = _stream_ptr(dev)
+        ws_bytes = lib.xattn_estimate_workspace_bytes(heads, q_len, k_len, stride, block_size, chunk_size, 0)
+        if ws_bytes == 0:
+            raise _hb.XattnHipError("estimator rejected the problem geometry")
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        sums = torch.empty((heads, nqb, nkb), dtype=torch.float32, device=dev)
+        scores = None
+        if dump_scores:
+            scores = torch.zeros(
+                (heads, (q_len + q_pad) // stride, (k_len + k_pad) // stride), dtype=torch.float32, device=dev
+            )
+        scale = 1.0 / math.sqrt(128) / stride / norm
+        _hb.check(
+            lib.xattn_estimate_block_sums(
+                q.data_ptr(), k.data_ptr(), sums.data_ptr(), workspace.data_ptr(), ws_bytes,
+                scores.data_ptr() if scores is not None else None,
+                heads, kv_heads, q_len, k_len, 128,
+                q.stride(1), q.stride(2), k.stride(1), k.stride(2),
+                stride, block_size, chunk_size, 0, q_chunks, int(bool(causal)), int(own_chunk_only),
+                scale, stream,
+            ),
+            "xattn_estimate_block_sums",
+        )
+        tau = _tau_per_head(threshold, heads, dev)
+        mask = torch.empty((heads, nqb, nkb), dtype=torch.uint8, device=dev)
+        col_idx = col_cnt = None
+        list_cols = (k_len + block_size - 1) // block_size
+        if want_lists:
+            col_idx = torch.empty((heads, nqb, list_cols), dtype=torch.int32, device=dev)
+            col_cnt = torch.empty((heads, nqb), dtype=torch.int32, device=dev)
+        _hb.check(
+            lib.xattn_select_blocks(
+                sums.data_ptr(), tau.data_ptr(), mask.data_ptr(),
+                col_idx.data_ptr() if want_lists else None,
+                col_cnt.data_ptr() if want_lists else None,
+                list_cols, heads, nqb, nkb, 0, nqb, nkb - nqb,
+                int(bool(causal)), int(bool(keep_sink)), int(bool(keep_recent)),
+                list_cols, q_len, k_len - q_len, stream,
+            ),
+            "xattn_select_blocks",
+        )
+    return dict(sums=sums, mask=mask, col_idx=col_idx, col_cnt=col_cnt, scores=scores, tau=tau)
+
+
+def xattn_estimate(
+    query_states,
+    key_states,
+    block_size,
+    stride,
+    norm=1,
+    softmax=True,
+    threshold=0.9,
+    chunk_size=16384,
+    select_mode="inverse",
+    use_triton=True,
+    causal=True,
+    kdb: int = 1,
+    keep_sink=False,
+    keep_recent=False,
+):
+    """Antidiagonal block scores and the thresholded block mask.
+
+    Same contract as xattn/src/Xattention.py:13-299: returns
+    ``(attn_sums, simple_masks)``, both ``[1, H, Nq_p, Nk_p]`` over the lengths
+    padded to multiples of ``chunk_size``; ``attn_sums`` in the query dtype,
+    ``simple_masks`` bool.  Only ``select_mode="inverse"``, ``kdb=1`` and
+    ``softmax=True`` (what every caller in the reference uses) are implemented.
+    """
+    if select_mode not in ("inverse", ""):
+        raise NotImplementedError(f"select_mode={select_mode!r} is not implemented on the HIP path")
+    if kdb != 1:
+        raise ValueError("kdb != 1 is not supported by the fused estimator")
+    if not softmax:
+        raise NotImplementedError("softmax=False is not implemented on the HIP path")
+    r = estimate_and_select(
+        query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
+        use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
+        want_lists=False,
+    )
+    attn_sums = r["sums"].to(query_states.dtype).unsqueeze(0)
+    simple_masks = r["mask"].view(torch.bool).unsqueeze(0)
+    return attn_sums, simple_masks
+
+
+def block_sparse_attention(query_states, key_states, value_states, col_idx=None, col_cnt=None,
+                           causal=True, softmax_scale=None):
+    """Attention of each 128-token query block over the key blocks listed for it
+    (``col_idx``/``col_cnt`` as written by :func:`estimate_and_select`; ``None``
+    visits every visible block = dense FlashAttention).  Stands in for
+    ``block_sparse_attn_func`` at xattn/src/Xattention.py:377-391.
+    Returns ``[1, H, q_len, 128]`` as a transposed view of ``[1, q_len, H, 128]``.
+    """
+    lib = _hb.lib()
+    q = _check_qk(query_states, "query_states")
+    k = _check_qk(key_states, "key_states")
+    v = _check_qk(value_states, "value_states")
+    dev = q.device
+    if k.device != dev:
+        k = k.to(dev)
+    if v.device != dev:
+        v = v.to(dev)
+    heads, q_len = q.shape[1], q.shape[2]
+    kv_heads, k_len = k.shape[1], k.shape[2]
+    if v.shape[1] != kv_heads or v.shape[2] != k_len:
+        raise AssertionError("key_states and value_states must agree in heads and length")
+    if (col_idx is None) != (col_cnt is None):
+        raise AssertionError("col_idx and col_cnt go together")
+    out = torch.empty((1, q_len, heads, 128), dtype=torch.bfloat16, device=dev)
+    scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(128)
+    if col_idx is not None:
+        assert col_idx.dtype == torch.int32 and col_cnt.dtype == torch.int32
+        assert col_idx.is_contiguous() and col_cnt.is_contiguous()
+        assert col_idx.shape[0] == heads and col_cnt.shape == col_idx.shape[:2]
+        pitch, idx_rows = col_idx.shape[2], col_idx.shape[1]
+    else:
+        pitch, idx_rows = 0, 0
+    with torch.cuda.device(dev):
+        _hb.check(
+            lib.xattn_block_sparse_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                col_idx.data_ptr() if col_idx is not None else None,
+                col_cnt.data_ptr() if col_cnt is not None else None,
+                pitch, idx_rows, heads, kv_heads, q_len, k_len, 128,
+                q.stride(1), q.stride(2), k.stride(1), k.stride(2), v.stride(1), v.stride(2),
+                out.stride(2), out.stride(1), int(bool(causal)), scale, _stream_ptr(dev),
+            ),
+            "xattn_block_sparse_fwd",
+        )
+    return out.transpose(1, 2)
+
+
+def Xattention_prefill(
+    query_states,
+    key_states,
+    value_states,
+    stride,
+    norm=1,
+    threshold=0.8,
+    block_size=128,
+    use_triton=True,
+    causal=True,
+    kdb=1,
+    chunk_size=None,
+    keep_sink=False,
+    keep_recent=False,
+):
+    """Sparse prefill attention: antidiagonal estimate -> block selection ->
+    block-sparse FlashAttention.  Signature, defaults and result layout of
+    xattn/src/Xattention.py:302-402."""
+    batch_size, _, k_len, _ = key_states.shape
+    assert block_size == 128
+    assert batch_size == 1
+    if kdb != 1:
+        raise ValueError("kdb != 1 is not supported by the fused estimator")
+    if chunk_size is None:
+        chunk_size = default_chunk_size(k_len)
+    r = estimate_and_select(
+        query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
+        use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
+        want_lists=True,
+    )
+    return block_sparse_attention(
+        query_states, key_states, value_states, r["col_idx"], r["col_cnt"], causal=causal
+    )
