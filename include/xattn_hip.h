@@ -95,7 +95,15 @@ int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, v
  * tau[h] * sum(row).  causal != 0: column 0 and the diagonal column
  * row + diag_offset are always kept; the remaining columns are visited by
  * descending block sum and kept while (forced mass + mass of those visited
- * before) < required; columns beyond the diagonal are cleared.  causal == 0:
+ * before) < required; columns beyond the diagonal are cleared (block sums there
+ * are taken as zero, which is what the estimator writes).  Rows are grouped
+ * into query chunks of blocks_per_chunk rows; in a chunk whose first diagonal is
+ * column 0 (diag_offset == 0 and row < blocks_per_chunk) the reference's eye()
+ * assignment overwrites the forced sink (utils.py:100-106) while its prefix
+ * still reserves two slots (utils.py:115-124): there only the diagonal is
+ * forced, the largest other block is always kept and each later one is judged
+ * against the mass gathered before its predecessor; column 0 ends up kept
+ * through the scatter of unselected ranks (utils.py:142).  causal == 0:
  * all columns are visited by descending block sum and kept while the mass
  * visited before is < required; if any column is left out, column 0 is kept
  * (utils.py:164).  keep_sink sets q-block row 0 entirely (Xattention.py:286-287);
@@ -111,7 +119,7 @@ int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uin
                         int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int num_heads,
                         int nq_blocks, int nk_blocks, int row_begin, int row_end, int diag_offset,
                         int causal, int keep_sink, int keep_recent, int list_cols, int q_len,
-                        int kv_off_tokens, void* stream);
+                        int kv_off_tokens, int blocks_per_chunk, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Block-sparse FlashAttention forward.  Replaces the call

@@ -30,7 +30,7 @@ def _select(sums, tau, causal, diag_offset, keep_sink=False, keep_recent=False):
         lib.xattn_select_blocks(
             s.data_ptr(), t.data_ptr(), mask.data_ptr(), idx.data_ptr(), cnt.data_ptr(), nk,
             H, nq, nk, 0, nq, diag_offset, int(causal), int(keep_sink), int(keep_recent),
-            nk, nq * 128, diag_offset * 128, torch.cuda.current_stream().cuda_stream,
+            nk, nq * 128, diag_offset * 128, nq, torch.cuda.current_stream().cuda_stream,
         ),
         "xattn_select_blocks",
     )
@@ -89,7 +89,7 @@ def test_keep_sink_and_keep_recent():
     got, idx, cnt = _select(x, 0.0, True, 0, keep_sink=True)
     assert got[:, 0, :].all()                       # row 0 entirely, future blocks included
     assert cnt[:, 0].tolist() == [1, 1]             # ... but the list holds visible blocks only
-    assert got[:, 1:].sum().item() == 2 * (7 * 2 - 0)
+    assert got[:, 1:].sum().item() == 2 * 7 * 2  # tau=0: sink + diagonal only
     xn = torch.rand(2, 8, 8, generator=g)
     got, _, _ = _select(xn, 0.2, False, 0, keep_recent=True)
     assert torch.diagonal(got, dim1=-2, dim2=-1).all()
@@ -121,7 +121,7 @@ def test_operator_mask_and_output_parity(name, L, H, Hkv, S, C, tau, causal, use
     )
     assert mask.dtype == torch.bool and mask.shape == want_mask.shape and sums.dtype == q.dtype
     off = 0
-    nbad, outside = mask_mismatch_report(want_sums[0], mask[0], want_mask[0], tau, causal, off)
+    nbad, outside = mask_mismatch_report(want_sums[0], mask[0], want_mask[0], tau, causal, off, C // 128)
     print(f"{name}: {nbad} mask mismatches, {outside} outside the tau band, density {want_mask.float().mean():.3f}")
     assert outside == 0
     assert nbad <= max(2, int(1e-3 * mask.numel()))

@@ -27,16 +27,18 @@ def test_golden_vectors_from_reference():
         assert torch.equal(got, c["mask"]), c["name"]
 
 
-def brute_select_row(vals, tau, causal, diag, limit):
+def brute_select_row(vals, tau, causal, diag, limit, first_diag=1):
     """Sorted-prefix enumeration for one row, written from the rule rather than
-    the tensor program: forced = {0, diag}; visit the rest by descending value
-    and keep a block while the mass gathered before it is below tau*total."""
+    the tensor program: forced = {0, diag} (only {diag} in a chunk whose first
+    diagonal is column 0, where eye() overwrites the sink, utils.py:100-106);
+    visit the rest by descending value and keep a block while the mass gathered
+    before it is below tau*total; unselected ranks land on column 0."""
     n = len(vals)
     total = sum(vals)
     need = total * tau
     keep = [False] * n
     if causal:
-        forced = sorted({0, diag})
+        forced = sorted({0, diag}) if first_diag != 0 else [diag]
         mass = 0.0
         for f in forced:
             keep[f] = True
@@ -48,6 +50,8 @@ def brute_select_row(vals, tau, causal, diag, limit):
             before = 0.0 if rank < extra else mass + sum(gathered[: rank - extra])
             if before < need:
                 keep[i] = True
+            else:
+                keep[0] = True  # scatter of unselected ranks, utils.py:142
             gathered.append(vals[i])
         for i in range(limit, n):
             keep[i] = False
@@ -66,11 +70,11 @@ def brute_select_row(vals, tau, causal, diag, limit):
     return keep
 
 
-@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("causal,cur", [(True, 8), (True, 0), (False, 0)])
 @pytest.mark.parametrize("tau", [0.0, 0.5, 0.9, 1.0])
-def test_bruteforce_enumeration(causal, tau):
-    g = torch.Generator().manual_seed(int(tau * 100) + causal)
-    rows, cols, cur = 6, 14, 8 if causal else 0
+def test_bruteforce_enumeration(causal, cur, tau):
+    g = torch.Generator().manual_seed(int(tau * 100) + causal + cur)
+    rows, cols = 6, 14
     x = torch.rand(1, 2, rows, cols, generator=g, dtype=torch.float64) + 0.01
     if causal:
         for r in range(rows):
@@ -79,8 +83,8 @@ def test_bruteforce_enumeration(causal, tau):
     for h in range(2):
         for r in range(rows):
             vals = x[0, h, r].tolist()
-            want = brute_select_row(vals, tau, causal, cur + r, cur + rows)
-            if causal and tau == 1.0:
+            want = brute_select_row(vals, tau, causal, cur + r, cur + rows, first_diag=cur)
+            if causal and (tau == 1.0 or cur == 0):
                 # zero-valued future blocks tie; compare only the causal part
                 want, have = want[: cur + r + 1], got[0, h, r, : cur + r + 1].tolist()
             else:

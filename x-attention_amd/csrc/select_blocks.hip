@@ -23,8 +23,15 @@ struct SelParams {
   int64_t idx_pitch;
   int H, nqb, nkb, row_begin, row_end, diag_offset;
   int causal, keep_sink, keep_recent, list_cols, q_len, kv_off;
+  int blocks_per_chunk;
   int npow2;   // LDS key capacity (power of two >= nkb)
 };
+
+// value encoded in a sort key (0 for forced blocks and padding)
+__device__ __forceinline__ double key_value(uint64_t key) {
+  const uint32_t hi = (uint32_t)(key >> 32);
+  return hi ? (double)__uint_as_float(hi - 1u) : 0.0;
+}
 
 __device__ __forceinline__ double wave_sum(double x) {
 #pragma unroll
@@ -43,6 +50,14 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   const int row = p.row_begin + blockIdx.x % rows;
   const float* x = p.sums + ((int64_t)head * p.nqb + row) * p.nkb;
   const int diag = row + p.diag_offset;
+  // Column index of the first diagonal of the row's query chunk.  When it is 0
+  // the reference's eye() assignment overwrites the forced sink column
+  // (utils.py:100-106), leaving the diagonal as the only forced block while
+  // the [0, forced_sum, ...] prefix (utils.py:115-124) still reserves two
+  // slots: the largest other block is then always kept and every later one is
+  // judged against the mass gathered before its predecessor.
+  const int chunk_first = p.diag_offset + (row / p.blocks_per_chunk) * p.blocks_per_chunk;
+  const bool one_forced = p.causal && chunk_first == 0;
 
   // candidates: columns [0, ncand); when causal nothing beyond the diagonal can be kept
   int ncand = p.nkb;
@@ -57,10 +72,11 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     if (c < ncand) {
       const float v = x[c];
       total += (double)v;
-      const bool forced = p.causal && (c == 0 || c == diag);
-      // block sums are >= 0, so their bit pattern orders like the value;
+      const bool forced = p.causal && (c == diag || (c == 0 && !one_forced));
+      // block sums are >= 0, so their bit pattern orders like the value (+1
+      // keeps every candidate ahead of the forced blocks, which sort last);
       // low word = ~column makes equal sums come out by ascending column
-      const uint32_t bits = forced ? 0u : __float_as_uint(v > 0.f ? v : 0.f);
+      const uint32_t bits = forced ? 0u : __float_as_uint(v > 0.f ? v : 0.f) + 1u;
       key = ((uint64_t)bits << 32) | (uint32_t)(~(uint32_t)c);
     }
     keys[c] = key;
@@ -70,7 +86,7 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   const double required = total * p.tau[head];
   double forced_sum = 0.0;
   if (p.causal && ncand > 0) {
-    forced_sum = (double)x[0];
+    if (!one_forced || diag == 0) forced_sum = (double)x[0];
     if (diag != 0 && diag < p.nkb) forced_sum += (double)x[diag];
   }
   __syncthreads();
@@ -95,7 +111,7 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   // fp64 exclusive prefix over the sorted values; rank kept while mass before it < required
   const int per = np2 >> 6;
   double local = 0.0;
-  for (int u = 0; u < per; ++u) local += (double)__uint_as_float((uint32_t)(keys[lane * per + u] >> 32));
+  for (int u = 0; u < per; ++u) local += key_value(keys[lane * per + u]);
   double incl = local;
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
@@ -105,14 +121,16 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   double before = forced_sum + (incl - local);
   int dropped = 0;
   for (int u = 0; u < per; ++u) {
-    const uint64_t key = keys[lane * per + u];
+    const int rank = lane * per + u;
+    const uint64_t key = keys[rank];
     const uint32_t col = ~(uint32_t)key;
-    if (col < (uint32_t)ncand) {
-      const bool forced = p.causal && ((int)col == 0 || (int)col == diag);
-      if (before < required) flags[col] = 1;
-      else if (!forced) dropped = 1;
+    if (col < (uint32_t)ncand && (key >> 32) != 0) {
+      double mass = before;
+      if (one_forced) mass = rank == 0 ? 0.0 : before - key_value(keys[rank - 1]);
+      if (mass < required) flags[col] = 1;
+      else dropped = 1;
     }
-    before += (double)__uint_as_float((uint32_t)(key >> 32));
+    before += key_value(key);
   }
   const bool any_dropped = __any(dropped);
   __syncthreads();
@@ -158,19 +176,21 @@ extern "C" int xattn_select_blocks(const float* block_sums, const double* tau_pe
                                    int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int num_heads,
                                    int nq_blocks, int nk_blocks, int row_begin, int row_end,
                                    int diag_offset, int causal, int keep_sink, int keep_recent,
-                                   int list_cols, int q_len, int kv_off_tokens, void* stream) {
+                                   int list_cols, int q_len, int kv_off_tokens, int blocks_per_chunk,
+                                   void* stream) {
   if (!block_sums || !tau_per_head || !mask) return XATTN_ERR_NULL;
   if ((col_idx == nullptr) != (col_cnt == nullptr)) return XATTN_ERR_NULL;
   if (num_heads <= 0 || nq_blocks <= 0 || nk_blocks <= 0 || nk_blocks > 16384) return XATTN_ERR_SHAPE;
   if (row_begin < 0 || row_end > nq_blocks || row_begin >= row_end) return XATTN_ERR_SHAPE;
   if (col_idx && idx_pitch < 1) return XATTN_ERR_SHAPE;
-  if (diag_offset < 0) return XATTN_ERR_SHAPE;
+  if (diag_offset < 0 || blocks_per_chunk < 1) return XATTN_ERR_SHAPE;
   SelParams p;
   p.sums = block_sums; p.tau = tau_per_head; p.mask = mask; p.col_idx = col_idx; p.col_cnt = col_cnt;
   p.idx_pitch = idx_pitch; p.H = num_heads; p.nqb = nq_blocks; p.nkb = nk_blocks;
   p.row_begin = row_begin; p.row_end = row_end; p.diag_offset = diag_offset;
   p.causal = causal ? 1 : 0; p.keep_sink = keep_sink ? 1 : 0; p.keep_recent = keep_recent ? 1 : 0;
   p.list_cols = list_cols; p.q_len = q_len; p.kv_off = kv_off_tokens;
+  p.blocks_per_chunk = blocks_per_chunk;
   int np2 = 64;
   while (np2 < nk_blocks) np2 <<= 1;
   p.npow2 = np2;

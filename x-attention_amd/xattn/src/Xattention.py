@@ -149,7 +149,7 @@ def estimate_and_select(
                 col_cnt.data_ptr() if want_lists else None,
                 list_cols, heads, nqb, nkb, 0, nqb, nkb - nqb,
                 int(bool(causal)), int(bool(keep_sink)), int(bool(keep_recent)),
-                list_cols, q_len, k_len - q_len, stream,
+                list_cols, q_len, k_len - q_len, chunk_size // block_size, stream,
             ),
             "xattn_select_blocks",
         )

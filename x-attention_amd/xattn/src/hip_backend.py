@@ -22,7 +22,7 @@ _SIGNATURES = {
     ),
     "xattn_select_blocks": (
         c_i32,
-        [c_vp] * 5 + [c_i64] + [c_i32] * 12 + [c_vp],
+        [c_vp] * 5 + [c_i64] + [c_i32] * 13 + [c_vp],
     ),
     "xattn_block_sparse_fwd": (
         c_i32,
