@@ -112,20 +112,21 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
 
-  // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD a
-  // contiguous slice of heads (so the KV heads it streams stay in its own L2)
-  // and hand out q-blocks from the last (longest, when causal) to the first.
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  Eight consecutive ids
+  // take eight consecutive q-blocks of ONE head, so every head's rows - whose
+  // list lengths vary smoothly with the row but by orders of magnitude between
+  // heads - are spread evenly over the XCDs; the next eight ids take the next
+  // head, so the query heads of a KV group with the same q-block run side by
+  // side on one XCD and share its L2 for K/V.  Rows go out last (longest, when
+  // causal) first.
   int head, qb;
   {
     const int id = blockIdx.x;
-    if (p.H % 8 == 0) {
-      const int hp = p.H / 8, x = id & 7, s = id >> 3;
-      head = x * hp + s % hp;
-      qb = p.nqb - 1 - s / hp;
-    } else {
-      head = id % p.H;
-      qb = p.nqb - 1 - id / p.H;
-    }
+    const int x = id & 7, s = id >> 3;
+    head = s % p.H;
+    const int from_end = (s / p.H) * 8 + x;
+    if (from_end >= p.nqb) return;
+    qb = p.nqb - 1 - from_end;
   }
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
@@ -308,7 +309,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   if (col_idx && (idx_pitch < 1 || idx_rows < p.nqb)) return XATTN_ERR_SHAPE;
   p.idx_rows = idx_rows;
 
-  const int64_t grid = (int64_t)p.H * p.nqb;
+  const int64_t grid = (int64_t)p.H * ((p.nqb + 7) / 8) * 8;
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
   hipLaunchKernelGGL(block_sparse_fwd_kernel, dim3((unsigned)grid), dim3(256), 0,
                      static_cast<hipStream_t>(stream), p);

@@ -39,6 +39,13 @@ def _stream_ptr(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def _mark(marks, label):
+    if marks is not None:
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        marks.append((label, ev))
+
+
 def _check_qk(x, name):
     if not x.is_cuda:
         raise _hb.XattnHipError(f"{name} must live on a ROCm device (no CPU fallback exists)")
@@ -80,8 +87,13 @@ def estimate_and_select(
     block_size=BLOCK,
     want_lists=True,
     dump_scores=False,
+    marks=None,
 ):
     """Runs the estimator and selection kernels.
+
+    ``marks``, when a list, receives ``(label, torch.cuda.Event)`` pairs recorded
+    on the current stream before the estimator, between estimator and selection
+    and after selection (for per-kernel timing).
 
     Returns a dict with fp32 ``sums`` [H, Nq_p, Nk_p], uint8 ``mask`` of the same
     shape, and (when ``want_lists``) ``col_idx`` [H, Nq_p, pitch] / ``col_cnt``
@@ -124,6 +136,7 @@ def estimate_and_select(
                 (heads, (q_len + q_pad) // stride, (k_len + k_pad) // stride), dtype=torch.float32, device=dev
             )
         scale = 1.0 / math.sqrt(128) / stride / norm
+        _mark(marks, "estimate_begin")
         _hb.check(
             lib.xattn_estimate_block_sums(
                 q.data_ptr(), k.data_ptr(), sums.data_ptr(), workspace.data_ptr(), ws_bytes,
@@ -136,6 +149,7 @@ def estimate_and_select(
             "xattn_estimate_block_sums",
         )
         tau = _tau_per_head(threshold, heads, dev)
+        _mark(marks, "select_begin")
         mask = torch.empty((heads, nqb, nkb), dtype=torch.uint8, device=dev)
         col_idx = col_cnt = None
         list_cols = (k_len + block_size - 1) // block_size
@@ -153,6 +167,7 @@ def estimate_and_select(
             ),
             "xattn_select_blocks",
         )
+        _mark(marks, "select_end")
     return dict(sums=sums, mask=mask, col_idx=col_idx, col_cnt=col_cnt, scores=scores, tau=tau)
 
 

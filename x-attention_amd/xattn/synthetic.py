@@ -4,13 +4,16 @@ The workloads are not taken from the reference (its benchmark needs model
 weights); they are defined here:
 
 * ``text`` tokens: q, k, v ~ N(0,1) per element.  A rank-8 term is then added to
-  both q and k: per token t a coefficient row a_t ~ N(0,1)^8 (shared by q and k
-  and by all heads), per KV head g a basis W_g ~ N(0,1)^{8 x d}; the term is
-  ``2.0 * a_t @ W_g / sqrt(8)`` (query head h uses the basis of its KV head).
-  Finally rotary position embedding, rotate-half form, base 500000, positions
-  0..L-1, on q and k.  Same-token q/k share the term (a strong block diagonal);
-  pairs with aligned coefficients give heavy off-diagonal entries whose
-  strength decays with distance through the rotary phases.
+  both q and k: with C ~ N(0,1)^{H_kv x 8} and B ~ N(0,1)^{8 x d}, the matrix of
+  per-head directions U = C B / sqrt(8) has rank 8; every token of KV head g -
+  its keys and the queries of the query heads that read it - gets ``2.0 * U[g]``
+  added.  Finally rotary position embedding, rotate-half form, base 500000,
+  positions 0..L-1, on q and k.  Before the rotation all queries and keys of a
+  head share the direction, so q.k carries a positive common term; the rotation
+  makes that term a function of the distance between the tokens, largest at
+  distance 0 and falling off roughly like a power of the distance whose
+  exponent grows with |U[g]|^2 - heads differ from sharply local to
+  heavy-tailed.  (The first key block is always kept by the selection rule.)
 * ``video`` tokens (workload 3): per frame of 256 tokens a mean vector ~ N(0,1)
   plus N(0, 0.3^2) per-token noise, drawn independently for q, k and v; the
   same rotary embedding on q and k.
@@ -98,7 +101,6 @@ def make_inputs(w: Workload, device="cpu", seed=0, L=None, heads=None, kv_heads=
     if w.kind == "field+text":
         T, Hh, Ww = 33, 45, 80
         n_field = T * Hh * Ww
-        scale = n_field / w.L
         if L != w.L:  # shrink the time axis for reduced-size runs
             T = max(1, int(round(T * L / w.L)))
             n_field = min(L, T * Hh * Ww)
@@ -125,13 +127,14 @@ def make_inputs(w: Workload, device="cpu", seed=0, L=None, heads=None, kv_heads=
     if w.kind == "video+text":
         frames = 240 if L == w.L else max(1, (L * 240 // w.L))
         n_video = min(L, frames * 256)
-    coeff = _randn((L, 8), gen, device)           # a_t, shared by q and k and all heads
-    basis = _randn((Hkv, 8, D), gen, device)      # W_g
+    coeff = _randn((Hkv, 8), gen, device)
+    basis = _randn((8, D), gen, device)
+    direction = 2.0 * (coeff @ basis) / math.sqrt(8.0)   # [Hkv, D], rank 8, shared by q and k
 
     def tokens(kv_head, shared):
         x = _randn((L, D), gen, device)
         if shared:
-            x[n_video:] += (2.0 / math.sqrt(8.0)) * (coeff[n_video:] @ basis[kv_head])
+            x[n_video:] += direction[kv_head]
         if n_video:
             nf = (n_video + 255) // 256
             means = _randn((nf, D), gen, device).repeat_interleave(256, dim=0)[:n_video]
