@@ -32,6 +32,7 @@ struct EstParams {
   const __bf16* q;
   const __bf16* k;
   int64_t q_sh, q_sn, k_sh, k_sn;
+  int64_t q_bytes, k_bytes;   // per-head extent q_len * q_sn * 2 (tokens beyond read as zeros)
   float* P;        // [H][nkb][rows]  partial block sums relative to the tile maximum
   float* Mt;       // [H][nT][rows]   tile maximum (exp2 domain)
   float* Lt;       // [H][nT][rows]   tile sum
@@ -46,6 +47,9 @@ struct EstParams {
   int real_rows;            // query rows >= real_rows are padding
   int causal, own_chunk_only;
   float scale_log2;
+  int nMT, nNT;             // tile rows over [row_begin, row_end) / tile columns over n_rk
+  int tiles_per_head;       // tiles with a visible pair, per head
+  int64_t total_tiles;      // tiles_per_head * H
 };
 
 // first / last visible reshaped key of reshaped query row m
@@ -56,38 +60,37 @@ __device__ __forceinline__ int row_hi(const EstParams& p, int m) {
   return p.causal ? m + p.off : p.n_rk - 1;
 }
 
-// One k-step slab: 256 rows x 64 bf16 per operand.  8 lanes fetch one row's
-// 128-byte line; tokens past the real length read as zeros (the padding of
-// xattn/src/Xattention.py:33-51).
-__device__ __forceinline__ void load_slab(const __bf16* base, int64_t sn, int len, int first_row, int S,
-                                          int tok_in_group, int feat0, int tid, u32x4 (&st)[8]) {
-  const int c = tid & 7, r0 = tid >> 3;
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int64_t tok = (int64_t)(first_row + r0 + 32 * it) * S + tok_in_group;
-    const bool ok = tok < len;
-    const u32x4 z = {0u, 0u, 0u, 0u};
-    u32x4 x = z;
-    if (ok) x = *reinterpret_cast<const u32x4*>(base + tok * sn + feat0 + c * 8);
-    st[it] = x;
-  }
-}
+// A k-step slab is 256 rows x 64 bf16 (one 128-byte line per row) per operand,
+// copied global -> LDS by buffer loads that write LDS directly (no register
+// staging): each wavefront instruction moves 64 x 16 bytes into one contiguous
+// KiB, i.e. 8 rows.  Tokens past the real length fall outside the buffer
+// resource and arrive as zeros - the zero padding of xattn/src/Xattention.py:33-51.
+//
+// LDS slab layout: row r at byte r*128; its 16-byte chunk c sits at position
+// c ^ (r & 7), so 8 lanes reading the same logical chunk of 8 consecutive rows
+// touch all banks.  The swizzle is applied on the global side of the copy
+// (the lane that fills position c fetches chunk c ^ (r & 7)).
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-// LDS slab layout: row r at byte r*128, its 16-byte chunk c stored at chunk
-// c ^ (r & 7) so that 8 lanes reading the same logical chunk of 8 consecutive
-// rows touch all banks.
-__device__ __forceinline__ void store_slab(char* slab, int tid, const u32x4 (&st)[8]) {
-  const int c = tid & 7, r0 = tid >> 3;
+__device__ __forceinline__ void copy_slab(__amdgpu_buffer_rsrc_t rsrc, int64_t sn_bytes, int first_row, int S,
+                                          int tok_in_group, int feat0_bytes, char* slab, int lane, int wave) {
+  const int c = lane & 7, rl = lane >> 3;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
-    const int r = r0 + 32 * it;
-    *reinterpret_cast<u32x4*>(slab + r * 128 + ((c ^ (r & 7)) << 4)) = st[it];
+    const int r = it * 32 + wave * 8 + rl;            // r & 7 == rl
+    const int64_t tok = (int64_t)(first_row + r) * S + tok_in_group;
+    int64_t off = tok * sn_bytes + feat0_bytes + ((c ^ rl) << 4);
+    off = off < 0x7fffffff ? off : 0x7fffffff;        // beyond every valid range -> zeros
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 32 + wave * 8) * 128), 16, (int)off, 0,
+                                             0, 0);
   }
 }
 
 __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk) {
   return *reinterpret_cast<const bf16x8*>(slab + row * 128 + ((chunk ^ (row & 7)) << 4));
 }
+
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 
 template <int RBS>
 __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
@@ -96,11 +99,40 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
-  const int head = blockIdx.z;
-  const int m0 = p.row_begin + blockIdx.y * kTile;
-  const int n0 = blockIdx.x * kTile;
+  // Tile assignment.  Only tiles holding a visible (row, key) pair are
+  // enumerated: per KV group, by query tile row, then key tile, then query head
+  // of the group.  Workgroup ids are dealt round-robin to the 8 XCDs, so runs of
+  // 32 consecutive tiles are given to one XCD: the 32 tiles an XCD works on at a
+  // time are then 8 key tiles x the heads of one group for one query tile row,
+  // which share their K' slabs across heads and their Q' slabs across key tiles
+  // in that XCD's L2, and every XCD gets the same number of tiles.
+  int head, m0, n0;
+  {
+    const int id = blockIdx.x;
+    const int64_t lin = ((int64_t)(id >> 8) * 8 + (id & 7)) * 32 + ((id >> 3) & 31);
+    if (lin >= p.total_tiles) return;
+    const int G = p.H / p.Hkv;
+    const int per_group = p.tiles_per_head * G;
+    const int g = (int)(lin / per_group);
+    int rem = (int)(lin % per_group);
+    head = g * G + rem % G;
+    int tt = rem / G;
+    int mt_row = 0, nt_first = 0;
+    for (;; ++mt_row) {
+      const int mfirst = p.row_begin + mt_row * kTile;
+      const int mlast = (mfirst + kTile - 1 < p.row_end ? mfirst + kTile - 1 : p.row_end - 1);
+      int hi = row_hi(p, mlast) / kTile;
+      hi = hi < p.nNT - 1 ? hi : p.nNT - 1;
+      nt_first = row_lo(p, mfirst) / kTile;
+      const int cnt = hi - nt_first + 1;
+      if (tt < cnt || mt_row + 1 >= p.nMT) break;
+      tt -= cnt;
+    }
+    m0 = p.row_begin + mt_row * kTile;
+    n0 = (nt_first + tt) * kTile;
+  }
 
-  // tiles without a visible (row, key) pair do nothing
+  // (kept as a guard) tiles without a visible (row, key) pair do nothing
   {
     const int m_last = (m0 + kTile - 1 < p.row_end ? m0 + kTile - 1 : p.row_end - 1);
     if (n0 > row_hi(p, m_last)) return;
@@ -110,6 +142,11 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+  const __amdgpu_buffer_rsrc_t qres =
+      __builtin_amdgcn_make_buffer_rsrc((void*)qbase, 0, (int)p.q_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t kres =
+      __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)p.k_bytes, 0x00020000);
+  const int64_t q_snb = p.q_sn * 2, k_snb = p.k_sn * 2;
 
   f32x16 acc[4][4];   // [key tile nt][query tile mt]
 #pragma unroll
@@ -120,41 +157,54 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
   const int steps = p.S * 2;
-  u32x4 stK[8], stQ[8];
-  load_slab(kbase, p.k_sn, p.Lk, n0, p.S, 0, 0, tid, stK);
-  load_slab(qbase, p.q_sn, p.Lq, m0, p.S, p.S - 1, 0, tid, stQ);
-  store_slab(lds, tid, stK);
-  store_slab(lds + kTile * 128, tid, stQ);
+  copy_slab(kres, k_snb, n0, p.S, 0, 0, lds, lane, wave);
+  copy_slab(qres, q_snb, m0, p.S, p.S - 1, 0, lds + kTile * 128, lane, wave);
+  wait_vm0();
   __syncthreads();
 
   for (int t = 0; t < steps; ++t) {
     char* cur = lds + (t & 1) * kStageBytes;
     char* nxt = lds + ((t + 1) & 1) * kStageBytes;
-    const bool more = t + 1 < steps;
-    if (more) {
-      const int i = (t + 1) >> 1, f0 = ((t + 1) & 1) * kDepth;
-      load_slab(kbase, p.k_sn, p.Lk, n0, p.S, i, f0, tid, stK);
-      load_slab(qbase, p.q_sn, p.Lq, m0, p.S, p.S - 1 - i, f0, tid, stQ);
+    if (t + 1 < steps) {
+      const int i = (t + 1) >> 1, f0 = ((t + 1) & 1) * kDepth * 2;
+      copy_slab(kres, k_snb, n0, p.S, i, f0, nxt, lane, wave);
+      copy_slab(qres, q_snb, m0, p.S, p.S - 1 - i, f0, nxt + kTile * 128, lane, wave);
     }
     const char* slabK = cur;
     const char* slabQ = cur + kTile * 128;
+    bf16x8 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      fa[0][x] = read_frag(slabK, wn * kSub + x * 32 + r, hh);
+      fb[0][x] = read_frag(slabQ, wm * kSub + x * 32 + r, hh);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);   // the first sub-step's 8 fragment reads
 #pragma unroll
     for (int ss = 0; ss < 4; ++ss) {
-      bf16x8 fa[4], fb[4];
+      if (ss < 3) {
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        fa[x] = read_frag(slabK, wn * kSub + x * 32 + r, ss * 2 + hh);
-        fb[x] = read_frag(slabQ, wm * kSub + x * 32 + r, ss * 2 + hh);
+        for (int x = 0; x < 4; ++x) {
+          fa[(ss + 1) & 1][x] = read_frag(slabK, wn * kSub + x * 32 + r, (ss + 1) * 2 + hh);
+          fb[(ss + 1) & 1][x] = read_frag(slabQ, wm * kSub + x * 32 + r, (ss + 1) * 2 + hh);
+        }
       }
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma32(fa[nt], fb[mt], acc[nt][mt]);
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma32(fa[ss & 1][nt], fb[ss & 1][mt], acc[nt][mt]);
+      // issue order: each LDS read of the NEXT sub-step's fragments is followed
+      // by two of this sub-step's MFMAs, so no MFMA waits on a read just issued
+      if (ss < 3) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 DS read
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
+        }
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+      }
     }
-    if (more) {
-      store_slab(nxt, tid, stK);
-      store_slab(nxt + kTile * 128, tid, stQ);
-    }
+    wait_vm0();
     __syncthreads();
   }
 
@@ -351,6 +401,10 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.q = static_cast<const __bf16*>(q);
   p.k = static_cast<const __bf16*>(k);
   p.q_sh = q_stride_h; p.q_sn = q_stride_n; p.k_sh = k_stride_h; p.k_sn = k_stride_n;
+  p.q_bytes = (int64_t)q_len * q_stride_n * 2;
+  p.k_bytes = (int64_t)k_len * k_stride_n * 2;
+  if (q_stride_n < kHeadDim || k_stride_n < kHeadDim) return XATTN_ERR_ALIGN;
+  if (p.q_bytes >= 0x7fffffff || p.k_bytes >= 0x7fffffff) return XATTN_ERR_SHAPE;
   p.H = num_heads; p.Hkv = num_kv_heads; p.Lq = q_len; p.Lk = k_len; p.S = stride;
   p.rbs = block_size / stride;
   p.n_rq = g.n_rq; p.n_rk = g.n_rk; p.nkb = g.nkb; p.nqb = g.nqb; p.nT = g.nT; p.rcs = g.rcs;
@@ -371,9 +425,23 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.Lt = p.Mt + (size_t)num_heads * g.nT * p.rows;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid1((g.n_rk + kTile - 1) / kTile, (p.rows + kTile - 1) / kTile, num_heads);
+  p.nMT = (p.rows + kTile - 1) / kTile;
+  p.nNT = (g.n_rk + kTile - 1) / kTile;
+  p.tiles_per_head = 0;
+  for (int r = 0; r < p.nMT; ++r) {   // same visibility rule as the kernel's row_lo / row_hi
+    const int mfirst = p.row_begin + r * kTile;
+    const int mlast = (mfirst + kTile - 1 < p.row_end ? mfirst + kTile - 1 : p.row_end - 1);
+    int hi = (p.causal ? mlast + p.off : p.n_rk - 1) / kTile;
+    hi = hi < p.nNT - 1 ? hi : p.nNT - 1;
+    const int lo = ((p.causal && p.own_chunk_only) ? (mfirst / p.rcs) * p.rcs + p.off : 0) / kTile;
+    p.tiles_per_head += hi - lo + 1;
+  }
+  p.total_tiles = (int64_t)p.tiles_per_head * num_heads;
+  const int64_t ids = (p.total_tiles + 255) / 256 * 256;
+  if (ids > 0x7fffffff) return XATTN_ERR_SHAPE;
+  const dim3 grid1((unsigned)ids);
   const dim3 grid2((p.rows + 63) / 64, num_heads);
-  if (grid1.y > 65535 || grid1.z > 65535 || grid2.y > 65535) return XATTN_ERR_SHAPE;
+  if (grid2.y > 65535) return XATTN_ERR_SHAPE;
   const size_t lds = 2 * (size_t)kStageBytes;
   hipError_t e = hipSuccess;
   switch (p.rbs) {
