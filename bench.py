@@ -85,6 +85,9 @@ def main():
     ap.add_argument("--workload", type=int, default=2, help="index into the synthetic workloads (default: headline)")
     ap.add_argument("--dense-steps", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) so that HBM byte "
+                         "counters collected over this command can be scaled by a kernel of known traffic")
     ap.add_argument("--seq-len", type=int, default=None, help="override L (debug only; invalidates the metric)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -202,6 +205,17 @@ def main():
         },
     }
     del dense, out
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        hip_backend.check(
+            hip_backend.lib().xattn_calibration_copy(
+                dst.data_ptr(), src.data_ptr(), src.numel() * 4, torch.cuda.current_stream().cuda_stream
+            ),
+            "xattn_calibration_copy",
+        )
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_cpu_baseline:
         base, (cq, ck, cv, cmask) = cpu_baseline()
         # the same sample on the GPU path (bf16), for scale

@@ -143,6 +143,13 @@ int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* ou
                            int64_t o_stride_h, int64_t o_stride_n, int causal, float softmax_scale,
                            void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Measurement aid, no counterpart in the reference: copies `bytes` (a multiple
+ * of 16) from src to dst with a plain kernel, i.e. reads `bytes` and writes
+ * `bytes` of HBM.  Profiling runs use it to scale hardware byte counters.
+ */
+int xattn_calibration_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,12 +38,13 @@ def _run(cmd):
 
 def build(verbose=True):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    extra = os.environ.get("XATTN_HIPCC_EXTRA", "").split()
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(HERE, s))]
     objs = [os.path.join(HERE, s.replace(".hip", ".o")) for s in srcs]
 
     def compile_one(pair):
         src, obj = pair
-        return _run([hipcc] + FLAGS + ["-c", src, "-o", obj])
+        return _run([hipcc] + FLAGS + extra + ["-c", src, "-o", obj])
 
     with ThreadPoolExecutor(max_workers=4) as ex:
         outs = list(ex.map(compile_one, zip(srcs, objs)))

@@ -72,18 +72,27 @@ __device__ __forceinline__ int row_hi(const EstParams& p, int m) {
 // (the lane that fills position c fetches chunk c ^ (r & 7)).
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-__device__ __forceinline__ void copy_slab(__amdgpu_buffer_rsrc_t rsrc, int64_t sn_bytes, int first_row, int S,
-                                          int tok_in_group, int feat0_bytes, char* slab, int lane, int wave) {
+// Per-lane byte offsets of the 8 rows a lane copies per slab, for token 0 of
+// each reshaped row's group and feature 0; the k-step adds a uniform term.
+// Offsets that do not fit 31 bits are pinned there: the host guarantees every
+// valid byte lies below 2^31, so they (and anything they grow into) read zeros.
+__device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int first_row, int S, int lane, int wave,
+                                             int (&voff)[8]) {
   const int c = lane & 7, rl = lane >> 3;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int r = it * 32 + wave * 8 + rl;            // r & 7 == rl
-    const int64_t tok = (int64_t)(first_row + r) * S + tok_in_group;
-    int64_t off = tok * sn_bytes + feat0_bytes + ((c ^ rl) << 4);
-    off = off < 0x7fffffff ? off : 0x7fffffff;        // beyond every valid range -> zeros
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 32 + wave * 8) * 128), 16, (int)off, 0,
-                                             0, 0);
+    const int64_t off = (int64_t)(first_row + r) * S * sn_bytes + ((c ^ rl) << 4);
+    voff[it] = off < 0x7fffffff ? (int)off : 0x7fffffff;
   }
+}
+
+__device__ __forceinline__ void copy_slab(__amdgpu_buffer_rsrc_t rsrc, const int (&voff)[8], int step_off,
+                                          char* slab, int wave) {
+#pragma unroll
+  for (int it = 0; it < 8; ++it)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 32 + wave * 8) * 128), 16,
+                                             (int)((unsigned)voff[it] + (unsigned)step_off), 0, 0, 0);
 }
 
 __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk) {
@@ -92,7 +101,8 @@ __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk
 
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 
-template <int RBS>
+// kDump: also write the raw scores (test / seam builds only; kept out of the production instantiation)
+template <int RBS, bool kDump>
 __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -157,8 +167,11 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
   const int steps = p.S * 2;
-  copy_slab(kres, k_snb, n0, p.S, 0, 0, lds, lane, wave);
-  copy_slab(qres, q_snb, m0, p.S, p.S - 1, 0, lds + kTile * 128, lane, wave);
+  int voffK[8], voffQ[8];
+  slab_offsets(k_snb, n0, p.S, lane, wave, voffK);
+  slab_offsets(q_snb, m0, p.S, lane, wave, voffQ);
+  copy_slab(kres, voffK, 0, lds, wave);
+  copy_slab(qres, voffQ, (p.S - 1) * (int)q_snb, lds + kTile * 128, wave);
   wait_vm0();
   __syncthreads();
 
@@ -167,8 +180,8 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
     char* nxt = lds + ((t + 1) & 1) * kStageBytes;
     if (t + 1 < steps) {
       const int i = (t + 1) >> 1, f0 = ((t + 1) & 1) * kDepth * 2;
-      copy_slab(kres, k_snb, n0, p.S, i, f0, nxt, lane, wave);
-      copy_slab(qres, q_snb, m0, p.S, p.S - 1 - i, f0, nxt + kTile * 128, lane, wave);
+      copy_slab(kres, voffK, i * (int)k_snb + f0, nxt, wave);
+      copy_slab(qres, voffQ, (p.S - 1 - i) * (int)q_snb + f0, nxt + kTile * 128, wave);
     }
     const char* slabK = cur;
     const char* slabQ = cur + kTile * 128;
@@ -215,12 +228,17 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
   float* Mst = p.Mt + ((int64_t)head * p.nT + T) * p.rows;
   float* Lst = p.Lt + ((int64_t)head * p.nT + T) * p.rows;
+  // every key of this wavefront tile visible to every one of its query rows?
+  // (true away from the diagonal and the sequence end: no per-element masking)
+  const int mw0 = m0 + wm * kSub;
+  const bool all_visible = nbase + kSub <= p.n_rk && nbase + kSub - 1 <= row_hi(p, mw0) &&
+                           nbase >= row_lo(p, mw0 + kSub - 1);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
     const int m = m0 + wm * kSub + mt * 32 + r;
     const bool row_ok = m < p.row_end;
     const int lo = row_lo(p, m), hi = row_hi(p, m);
-    if (p.scores && row_ok) {
+    if (kDump && row_ok) {
       float* dst = p.scores + ((int64_t)head * p.n_rq + m) * p.n_rk;
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
@@ -230,17 +248,24 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
           if (n < p.n_rk) dst[n] = acc[nt][mt][v];
         }
     }
-    float x[4][16];
+    // pass 1: row maximum over this tile's visible keys (exp2 domain)
     float mx = -INFINITY;
+    if (all_visible) {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int n = nbase + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
-        const bool vis = n >= lo && n <= hi && n < p.n_rk;
-        x[nt][v] = vis ? acc[nt][mt][v] * p.scale_log2 : -INFINITY;
-        mx = fmaxf(mx, x[nt][v]);
-      }
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc[nt][mt][v]);
+      mx *= p.scale_log2;   // scale > 0
+    } else {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int n = nbase + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
+          const bool vis = n >= lo && n <= hi && n < p.n_rk;
+          mx = fmaxf(mx, vis ? acc[nt][mt][v] * p.scale_log2 : -INFINITY);
+        }
+    }
     mx = fmaxf(mx, swap_half(mx));
     const float safe = (mx == -INFINITY) ? 0.f : mx;
     float tot = 0.f;
@@ -253,7 +278,15 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
       for (int g = 0; g < 4; ++g) {
         float s = 0.f;
 #pragma unroll
-        for (int t2 = 0; t2 < 4; ++t2) s += fast_exp2(x[nt][g * 4 + t2] - safe);
+        for (int t2 = 0; t2 < 4; ++t2) {
+          const int v = g * 4 + t2;
+          float e = fast_exp2(__builtin_fmaf(acc[nt][mt][v], p.scale_log2, -safe));
+          if (!all_visible) {
+            const int n = nbase + nt * 32 + g * 8 + hh * 4 + t2;
+            e = (n >= lo && n <= hi && n < p.n_rk) ? e : 0.f;
+          }
+          s += e;
+        }
         part[g] = s + swap_half(s);
         tot += part[g];
       }
@@ -280,6 +313,9 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
       Mst[mrel] = mx;
       Lst[mrel] = tot;
     }
+    // keep the four query-tile passes apart: interleaving them only lengthens
+    // live ranges on top of the 256 accumulator registers
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
@@ -344,6 +380,16 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
 using namespace xattn;
 
 namespace {
+template <int RBS>
+hipError_t launch_gemm(const EstParams& p, dim3 grid, size_t lds, hipStream_t s) {
+  auto kernel = p.scores ? &estimate_gemm_kernel<RBS, true> : &estimate_gemm_kernel<RBS, false>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kernel, grid, dim3(256), lds, s, p);
+  return hipSuccess;
+}
+
 struct Geometry {
   int q_pad, k_pad, n_rq, n_rk, nqb, nkb, nT, rcs, q_chunks;
 };
@@ -446,24 +492,18 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   hipError_t e = hipSuccess;
   switch (p.rbs) {
     case 8:
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&estimate_gemm_kernel<8>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      e = launch_gemm<8>(p, grid1, lds, s);
       if (e != hipSuccess) return XATTN_ERR_LAUNCH;
-      hipLaunchKernelGGL(estimate_gemm_kernel<8>, grid1, dim3(256), lds, s, p);
       hipLaunchKernelGGL(estimate_normalize_kernel<8>, grid2, dim3(256), 0, s, p);
       break;
     case 16:
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&estimate_gemm_kernel<16>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      e = launch_gemm<16>(p, grid1, lds, s);
       if (e != hipSuccess) return XATTN_ERR_LAUNCH;
-      hipLaunchKernelGGL(estimate_gemm_kernel<16>, grid1, dim3(256), lds, s, p);
       hipLaunchKernelGGL(estimate_normalize_kernel<16>, grid2, dim3(256), 0, s, p);
       break;
     default:
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&estimate_gemm_kernel<32>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      e = launch_gemm<32>(p, grid1, lds, s);
       if (e != hipSuccess) return XATTN_ERR_LAUNCH;
-      hipLaunchKernelGGL(estimate_gemm_kernel<32>, grid1, dim3(256), lds, s, p);
       hipLaunchKernelGGL(estimate_normalize_kernel<32>, grid2, dim3(256), 0, s, p);
       break;
   }
