@@ -12,18 +12,25 @@
 // wavefront owns 32 query rows.  Scores are produced transposed,
 // S^T = K Q^T, so that one lane owns one query row (softmax statistics need a
 // single cross-lane exchange) and the fp32 accumulator registers of S^T are,
-// unchanged, the B operand of O^T += V^T P^T.  K is staged row-major and V
-// transposed (with the accumulator's row permutation folded in) through LDS;
-// the next tile's global loads are in flight while the current one is
-// multiplied.  Two workgroups fit per CU (68 KiB LDS each) so one's softmax
-// overlaps the other's MFMA.
+// unchanged, the B operand of O^T += V^T P^T.  K and V tiles (128 keys x 128
+// features, row-major, XOR-swizzled 16-byte chunks) are copied global -> LDS by
+// buffer loads that write LDS directly; keys past the sequence end fall outside
+// the buffer resource and arrive as zeros.  K fragments are read with
+// ds_read_b128, V^T fragments with the transposing ds_read_b64_tr_b16, both
+// issued one k-step ahead of the MFMAs that consume them.  The copy of the next
+// K tile overlaps softmax and P.V, the copy of the next V tile overlaps Q.K^T.
+// Two workgroups fit per CU (64 KiB LDS each) so one's softmax overlaps the
+// other's MFMA.
 #include "xattn_common.h"
 #include "xattn_hip.h"
 
 namespace xattn {
 
 constexpr int kBlk = 128;          // block_size of the operator
-constexpr int kLdsRow = 136;       // bf16 per LDS row: 128 + 8 pad (272 B) -> conflict-free b128 reads
+constexpr int kTileBytes = kBlk * 256;   // one K or V tile in LDS
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4;
 
 struct AttnParams {
   const __bf16* q;
@@ -31,8 +38,8 @@ struct AttnParams {
   const __bf16* v;
   __bf16* o;
   int64_t q_sh, q_sn, k_sh, k_sn, v_sh, v_sn, o_sh, o_sn;  // element strides (head, token)
-  const int32_t* col_idx;   // [H, nqb, idx_pitch] ascending k-block ids, or null = all visible
-  const int32_t* col_cnt;   // [H, nqb]
+  const int32_t* col_idx;   // [H, idx_rows, idx_pitch] ascending k-block ids, or null = all visible
+  const int32_t* col_cnt;   // [H, idx_rows]
   int64_t idx_pitch;
   int idx_rows;             // q-block rows per head in col_idx / col_cnt (>= nqb)
   int H, Hkv, Lq, Lk, nqb, nkb;
@@ -42,74 +49,41 @@ struct AttnParams {
 
 __device__ __forceinline__ int clamp_block(int kb, int nkb) { return kb < 0 ? 0 : (kb < nkb ? kb : nkb - 1); }
 
-__device__ __forceinline__ void load_k_tile(const AttnParams& p, const __bf16* kbase, int kb, int tid,
-                                            u32x4 (&st)[8]) {
-  const int chunk = tid & 15, row0 = tid >> 4;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int n = kb * kBlk + i * 16 + row0;
-    n = n < p.Lk ? n : p.Lk - 1;   // rows past the end are masked in the softmax
-    st[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)n * p.k_sn + chunk * 8);
-  }
-}
+// LDS tile layout: row n at byte n*256, its 16-byte chunk c stored at chunk
+// c ^ swz(n).  swz takes all 16 values over 16 consecutive rows (row-per-lane
+// b128 reads of one logical chunk are conflict-free) and moves rows n..n+3 into
+// different 64-byte groups (the 4-row x 32-byte gathers of the transposing read
+// are conflict-free too).
+__device__ __forceinline__ int swz(int n) { return ((n & 3) << 2) | ((n >> 2) & 3); }
 
-__device__ __forceinline__ void store_k_tile(__bf16* Ks, int tid, const u32x4 (&st)[8]) {
-  const int chunk = tid & 15, row0 = tid >> 4;
+// Copies key block kb of one head (row stride sn elements) into an LDS tile.
+// Wavefront w issues 8 instructions of 1 KiB (4 rows) each; voff[i] is the
+// lane's byte offset inside the block for instruction i.
+__device__ __forceinline__ void copy_tile(const __bf16* base, int64_t sn, int len, int kb, const int (&voff)[8],
+                                          char* tile, int wave) {
+  const int rows_left = len - kb * kBlk;
+  const int rows = rows_left < kBlk ? rows_left : kBlk;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(base + (int64_t)kb * kBlk * sn), 0, (int)((int64_t)rows * sn * 2), 0x00020000);
 #pragma unroll
   for (int i = 0; i < 8; ++i)
-    *reinterpret_cast<u32x4*>(Ks + (i * 16 + row0) * kLdsRow + chunk * 8) = st[i];
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(tile + (wave * 8 + i) * 1024), 16, voff[i], 0, 0, 0);
 }
 
-// thread -> (4 consecutive key rows) x (8 consecutive features), twice
-__device__ __forceinline__ void load_v_tile(const AttnParams& p, const __bf16* vbase, int kb, int tid,
-                                            u32x4 (&st)[8]) {
-  const int lane = tid & 63, wave = tid >> 6;
-  const int ng = lane & 15, dc = (lane >> 4) + 4 * wave;
+__device__ __forceinline__ void tile_offsets(int64_t sn, int lane, int wave, int (&voff)[8]) {
 #pragma unroll
-  for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int n = kb * kBlk + hf * 64 + ng * 4 + i;
-      bool ok = n < p.Lk;
-      n = ok ? n : p.Lk - 1;
-      u32x4 x = *reinterpret_cast<const u32x4*>(vbase + (int64_t)n * p.v_sn + dc * 8);
-      const u32x4 z = {0u, 0u, 0u, 0u};
-      st[hf * 4 + i] = ok ? x : z;   // rows past the sequence end must be exact zeros
-    }
-}
-
-// Writes V^T: LDS row = feature, column = key position permuted so that the 8
-// keys one MFMA lane needs (n = 16s + 8a + 4h + t -> 16s + 8h + 4a + t) are
-// contiguous.
-__device__ __forceinline__ void store_v_tile_t(__bf16* Vt, int tid, const u32x4 (&st)[8]) {
-  const int lane = tid & 63, wave = tid >> 6;
-  const int ng = lane & 15, dc = (lane >> 4) + 4 * wave;
-#pragma unroll
-  for (int hf = 0; hf < 2; ++hf) {
-    const int n0 = hf * 64 + ng * 4;
-    const int pos = (n0 & ~15) + ((n0 >> 2) & 1) * 8 + ((n0 >> 3) & 1) * 4;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      uint32_t a = st[hf * 4 + 0][j >> 1], b = st[hf * 4 + 1][j >> 1];
-      uint32_t c = st[hf * 4 + 2][j >> 1], d = st[hf * 4 + 3][j >> 1];
-      u32x2 w;
-      if (j & 1) {
-        w[0] = (a >> 16) | (b & 0xffff0000u);
-        w[1] = (c >> 16) | (d & 0xffff0000u);
-      } else {
-        w[0] = (a & 0xffffu) | (b << 16);
-        w[1] = (c & 0xffffu) | (d << 16);
-      }
-      *reinterpret_cast<u32x2*>(Vt + (dc * 8 + j) * kLdsRow + pos) = w;
-    }
+  for (int i = 0; i < 8; ++i) {
+    const int row = 4 * (wave * 8 + i) + (lane >> 4);
+    const int c = (lane & 15) ^ swz(row);
+    voff[i] = (int)(row * sn * 2) + (c << 4);
   }
 }
 
 // kHasList = false is the dense baseline (its own symbol, so profiles tell the two apart)
 template <bool kHasList>
 __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) {
-  __shared__ __attribute__((aligned(16))) __bf16 Ks[kBlk * kLdsRow];
-  __shared__ __attribute__((aligned(16))) __bf16 Vt[kBlk * kLdsRow];
+  __shared__ __attribute__((aligned(1024))) char Ks[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) char Vs[kTileBytes];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
@@ -138,14 +112,17 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   const int q_row = qb * kBlk + wave * 32 + r;          // this lane's query token
   const int q_pos = q_row + p.kv_off;                   // its position on the key axis
   int n_blocks;
-  const int32_t* list = nullptr;
+  // the column list is read through the scalar cache (uniform, read-only), so that
+  // fetching the next block id never waits on the tile copies in flight
+  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+  const_i32_ptr list = nullptr;
   {
     const int q_last = (qb * kBlk + kBlk - 1 < p.Lq ? qb * kBlk + kBlk - 1 : p.Lq - 1) + p.kv_off;
     int visible = p.causal ? (q_last < 0 ? 0 : q_last / kBlk + 1) : p.nkb;
     visible = visible < p.nkb ? visible : p.nkb;
     if (kHasList) {
-      list = p.col_idx + ((int64_t)head * p.idx_rows + qb) * p.idx_pitch;
-      n_blocks = p.col_cnt[head * p.idx_rows + qb];
+      list = (const_i32_ptr)(uintptr_t)(p.col_idx + ((int64_t)head * p.idx_rows + qb) * p.idx_pitch);
+      n_blocks = ((const_i32_ptr)(uintptr_t)p.col_cnt)[head * p.idx_rows + qb];
       n_blocks = n_blocks < 0 ? 0 : (n_blocks > p.idx_pitch ? (int)p.idx_pitch : n_blocks);
     } else {
       n_blocks = visible;
@@ -161,6 +138,31 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(src + s * 16);
   }
 
+  // loop-invariant addressing
+  int voffK[8], voffV[8];
+  tile_offsets(p.k_sn, lane, wave, voffK);
+  tile_offsets(p.v_sn, lane, wave, voffV);
+  // K fragment (k-step s, key tile nt): row nt*32 + r, logical chunk 2s + hh
+  int kaddr[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) kaddr[s] = r * 256 + (((2 * s + hh) ^ swz(r)) << 4);
+  // V^T fragment (k-step ks, half a, feature tile dt): the transposing read hands
+  // lane l the feature dt*32 + (l % 32) of keys 16ks + 8a + 4hh + {0..3}; as a
+  // source lane it points at key e = (l%16)/4 of that quad, features
+  // dt*32 + 16*((l/16)%2) + 4*(l%4) .. +3.
+  int vaddr[4][2];
+  {
+    const int e = (lane & 15) >> 2, j = lane & 3, g2 = (lane >> 4) & 1;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        const int row = 8 * a + 4 * hh + e;                       // + 16*ks
+        const int c = dt * 4 + 2 * g2 + (j >> 1);
+        vaddr[dt][a] = row * 256 + ((c ^ swz(row)) << 4) + (j & 1) * 8;
+      }
+  }
+
   f32x16 oacc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -169,20 +171,17 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   float m_run = -INFINITY;   // running row maximum, already multiplied by scale_log2
   float l_run = 0.f;         // this lane's share of the running row sum
 
-  u32x4 stage[8];
   int kb = 0;
   if (n_blocks > 0) {
     kb = kHasList ? clamp_block(list[0], p.nkb) : 0;
-    load_k_tile(p, kbase, kb, tid, stage);
-    store_k_tile(Ks, tid, stage);
-    load_v_tile(p, vbase, kb, tid, stage);
+    copy_tile(kbase, p.k_sn, p.Lk, kb, voffK, Ks, wave);
+    copy_tile(vbase, p.v_sn, p.Lk, kb, voffV, Vs, wave);
   }
+  wait_vm0();
+  __syncthreads();                         // K_0 (and V_0) landed and visible
 
   for (int j = 0; j < n_blocks; ++j) {
     const int kb_next = (j + 1 < n_blocks) ? (kHasList ? clamp_block(list[j + 1], p.nkb) : j + 1) : -1;
-    __syncthreads();                       // K_j visible in Ks; everyone is done with V_{j-1}
-    store_v_tile_t(Vt, tid, stage);
-    if (kb_next >= 0) load_k_tile(p, kbase, kb_next, tid, stage);
 
     // ---- S^T = K_j Q^T : lane owns query row r, key rows 8g + 4hh + t of each 32-row tile
     f32x16 sacc[4];
@@ -190,13 +189,34 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) sacc[i][v] = 0.f;
+    {
+      bf16x8 kf[2][4];
 #pragma unroll
-    for (int s = 0; s < 8; ++s)
+      for (int nt = 0; nt < 4; ++nt) kf[0][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[0] + nt * 8192);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        bf16x8 a = *reinterpret_cast<const bf16x8*>(Ks + (nt * 32 + r) * kLdsRow + s * 16 + hh * 8);
-        sacc[nt] = mfma32(a, qreg[s], sacc[nt]);
+      for (int s = 0; s < 8; ++s) {
+        if (s < 7) {
+#pragma unroll
+          for (int nt = 0; nt < 4; ++nt)
+            kf[(s + 1) & 1][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[s + 1] + nt * 8192);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) sacc[nt] = mfma32(kf[s & 1][nt], qreg[s], sacc[nt]);
+        if (s < 7) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          }
+        } else {
+          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        }
       }
+    }
+    wait_vm0();
+    __syncthreads();                       // everyone is done with K_j; V_j landed and visible
+    if (kb_next >= 0) copy_tile(kbase, p.k_sn, p.Lk, kb_next, voffK, Ks, wave);
 
     const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
     if (need_mask) {
@@ -237,20 +257,51 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
 #pragma unroll
       for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
 
-    __syncthreads();                       // V_j^T visible in Vt; everyone is done with K_j
-    if (kb_next >= 0) {
-      store_k_tile(Ks, tid, stage);
-      load_v_tile(p, vbase, kb_next, tid, stage);
-    }
-
     // ---- O^T += V_j^T P^T
+    {
+      i16x4 vf[2][4][2];
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
+      for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        bf16x8 a = *reinterpret_cast<const bf16x8*>(Vt + (dt * 32 + r) * kLdsRow + ks * 16 + hh * 8);
-        oacc[dt] = mfma32(a, pfrag[ks], oacc[dt]);
+        for (int a = 0; a < 2; ++a)
+          vf[0][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a]));
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        if (ks < 7) {
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+              vf[(ks + 1) & 1][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                  (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a] + (ks + 1) * 4096));
+        }
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+          typedef __attribute__((__vector_size__(8 * sizeof(short)))) short i16x8;
+          i16x8 av;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            av[u] = vf[ks & 1][dt][0][u];
+            av[4 + u] = vf[ks & 1][dt][1][u];
+          }
+          oacc[dt] = mfma32(__builtin_bit_cast(bf16x8, av), pfrag[ks], oacc[dt]);
+        }
+        if (ks < 7) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          }
+        } else {
+          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        }
       }
+    }
+    wait_vm0();
+    __syncthreads();                       // everyone is done with V_j; K_{j+1} landed and visible
+    if (kb_next >= 0) copy_tile(vbase, p.v_sn, p.Lk, kb_next, voffV, Vs, wave);
     kb = kb_next;
   }
 

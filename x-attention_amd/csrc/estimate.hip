@@ -99,7 +99,6 @@ __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk
   return *reinterpret_cast<const bf16x8*>(slab + row * 128 + ((chunk ^ (row & 7)) << 4));
 }
 
-__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 
 // kDump: also write the raw scores (test / seam builds only; kept out of the production instantiation)
 template <int RBS, bool kDump>

@@ -33,6 +33,10 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, p);
 }
 
+// waits until every outstanding global/buffer load of this wavefront (including
+// loads that write LDS directly) has completed; LDS and scalar counters untouched
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // value held by the lane 32 positions away (the other half-wave)
 __device__ __forceinline__ float swap_half(float x) { return __shfl_xor(x, 32, 64); }
 
