@@ -67,9 +67,10 @@ __device__ __forceinline__ int row_hi(const EstParams& p, int m) {
 // resource and arrive as zeros - the zero padding of xattn/src/Xattention.py:33-51.
 //
 // LDS slab layout: row r at byte r*128; its 16-byte chunk c sits at position
-// c ^ (r & 7), so 8 lanes reading the same logical chunk of 8 consecutive rows
-// touch all banks.  The swizzle is applied on the global side of the copy
-// (the lane that fills position c fetches chunk c ^ (r & 7)).
+// c ^ ((r >> 1) & 7), so the 16 lanes of one ds_read_b128 pass - the same
+// logical chunk of 16 consecutive rows - touch each of the 64 banks once.  The
+// swizzle is applied on the global side of the copy (the lane that fills
+// position c fetches chunk c ^ ((r >> 1) & 7)).
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // Per-lane byte offsets of the 8 rows a lane copies per slab, for token 0 of
@@ -81,8 +82,8 @@ __device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int first_row, in
   const int c = lane & 7, rl = lane >> 3;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
-    const int r = it * 32 + wave * 8 + rl;            // r & 7 == rl
-    const int64_t off = (int64_t)(first_row + r) * S * sn_bytes + ((c ^ rl) << 4);
+    const int r = it * 32 + wave * 8 + rl;
+    const int64_t off = (int64_t)(first_row + r) * S * sn_bytes + ((c ^ ((r >> 1) & 7)) << 4);
     voff[it] = off < 0x7fffffff ? (int)off : 0x7fffffff;
   }
 }
@@ -96,7 +97,7 @@ __device__ __forceinline__ void copy_slab(__amdgpu_buffer_rsrc_t rsrc, const int
 }
 
 __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk) {
-  return *reinterpret_cast<const bf16x8*>(slab + row * 128 + ((chunk ^ (row & 7)) << 4));
+  return *reinterpret_cast<const bf16x8*>(slab + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
 }
 
 
