@@ -1,0 +1,67 @@
+"""The C-ABI library loads without a GPU and exports every function that
+include/xattn_hip.h declares; the ctypes binding covers the same set."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "xattn_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(xattn_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("xattn_estimate_block_sums", "xattn_select_blocks", "xattn_block_sparse_fwd",
+                 "xattn_estimate_workspace_bytes", "xattn_abi_version", "xattn_error_string"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from xattn.src import hip_backend as hb
+
+    if not os.path.exists(hb.LIB_PATH):
+        pytest.fail(f"{hb.LIB_PATH} has not been built (python x-attention_amd/csrc/build.py)")
+    lib = ctypes.CDLL(hb.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    assert sorted(hb.exported_symbols()) == declared_functions()
+
+
+def test_host_side_calls_need_no_gpu():
+    from xattn.src import hip_backend as hb
+
+    lib = hb.lib()
+    assert lib.xattn_abi_version() >= 1
+    assert lib.xattn_error_string(0) == b"ok"
+    assert b"128" in lib.xattn_error_string(-2)
+    # geometry helper: pure host arithmetic
+    assert lib.xattn_estimate_workspace_bytes(32, 131072, 131072, 16, 128, 16384, 0) == 32 * 8192 * (1024 + 2 * 64) * 4
+    assert lib.xattn_estimate_workspace_bytes(32, 131072, 131072, 3, 128, 16384, 0) == 0     # bad stride
+    assert lib.xattn_estimate_workspace_bytes(32, 4096, 2048, 8, 128, 2048, 0) == 0          # k shorter than q
+
+
+def test_operator_refuses_cpu_tensors_and_wrong_dtypes():
+    import torch
+
+    from xattn.src import hip_backend as hb
+    from xattn.src.Xattention import Xattention_prefill, default_chunk_size, xattn_estimate
+
+    q = torch.zeros(1, 2, 256, 128, dtype=torch.bfloat16)
+    with pytest.raises(hb.XattnHipError):
+        Xattention_prefill(q, q, q, 8)
+    with pytest.raises(NotImplementedError):
+        xattn_estimate(q, q, 128, 8, select_mode="slash")
+    with pytest.raises(ValueError):
+        xattn_estimate(q, q, 128, 8, kdb=2)
+    with pytest.raises(NotImplementedError):
+        xattn_estimate(q, q, 128, 8, softmax=False)
+    table = {1024: 2048, 4096: 4096, 16384: 16384, 32768: 8192, 65536: 4096, 131072: 2048, 119056: 2048}
+    for L, want in table.items():
+        assert default_chunk_size(L) == want
