@@ -26,6 +26,9 @@ for _p in (ROOT, os.path.join(ROOT, "x-attention_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs whose summary is
+# kept under profiles/ (counters cannot be read from inside this process); other workloads report null.
+MEASURED_TRAFFIC_BYTES = {"cfg2_llama8b_L131072_gqa32x8_S16": 2.019e10}
 
 
 def _ms(a, b):
@@ -201,7 +204,7 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(sparse_tflops / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name) if L == w.L else None,
         },
     }
     del dense, out
