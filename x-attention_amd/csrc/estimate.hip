@@ -96,6 +96,12 @@ __device__ __forceinline__ void copy_slab(__amdgpu_buffer_rsrc_t rsrc, const int
                                              (int)((unsigned)voff[it] + (unsigned)step_off), 0, 0, 0);
 }
 
+__device__ __forceinline__ void copy_one(__amdgpu_buffer_rsrc_t rsrc, int voff, int step_off, char* slab, int wave,
+                                         int it) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 32 + wave * 8) * 128), 16,
+                                           (int)((unsigned)voff + (unsigned)step_off), 0, 0, 0);
+}
+
 __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk) {
   return *reinterpret_cast<const bf16x8*>(slab + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4));
 }
@@ -178,11 +184,11 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   for (int t = 0; t < steps; ++t) {
     char* cur = lds + (t & 1) * kStageBytes;
     char* nxt = lds + ((t + 1) & 1) * kStageBytes;
-    if (t + 1 < steps) {
-      const int i = (t + 1) >> 1, f0 = ((t + 1) & 1) * kDepth * 2;
-      copy_slab(kres, voffK, i * (int)k_snb + f0, nxt, wave);
-      copy_slab(qres, voffQ, (p.S - 1 - i) * (int)q_snb + f0, nxt + kTile * 128, wave);
-    }
+    // the last step copies its own slabs again into the idle stage, which keeps
+    // the loop body free of branches
+    const int tn = t + 1 < steps ? t + 1 : t;
+    const int offK = (tn >> 1) * (int)k_snb + (tn & 1) * kDepth * 2;
+    const int offQ = (p.S - 1 - (tn >> 1)) * (int)q_snb + (tn & 1) * kDepth * 2;
     const char* slabK = cur;
     const char* slabQ = cur + kTile * 128;
     bf16x8 fa[2][4], fb[2][4];
@@ -191,32 +197,32 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
       fa[0][x] = read_frag(slabK, wn * kSub + x * 32 + r, hh);
       fb[0][x] = read_frag(slabQ, wm * kSub + x * 32 + r, hh);
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);   // the first sub-step's 8 fragment reads
+    // The step is cut into 16 chunks that the scheduler may not mix: one of the
+    // 16 copies of the next k-step, two of the 8 fragment reads of the next
+    // sub-step, four MFMAs.  With one wavefront per SIMD issue is in order, so a
+    // burst of copies or reads would hold back the MFMAs queued behind it.
 #pragma unroll
     for (int ss = 0; ss < 4; ++ss) {
-      if (ss < 3) {
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
-          fa[(ss + 1) & 1][x] = read_frag(slabK, wn * kSub + x * 32 + r, (ss + 1) * 2 + hh);
-          fb[(ss + 1) & 1][x] = read_frag(slabQ, wm * kSub + x * 32 + r, (ss + 1) * 2 + hh);
+      for (int c = 0; c < 4; ++c) {
+        __builtin_amdgcn_sched_barrier(0);
+        const int it = ss * 2 + (c >> 1);
+        if (c & 1) copy_one(qres, voffQ[it], offQ, nxt + kTile * 128, wave, it);
+        else copy_one(kres, voffK[it], offK, nxt, wave, it);
+        if (ss < 3) {
+          if (c < 2) {
+            fa[(ss + 1) & 1][2 * c] = read_frag(slabK, wn * kSub + (2 * c) * 32 + r, (ss + 1) * 2 + hh);
+            fa[(ss + 1) & 1][2 * c + 1] = read_frag(slabK, wn * kSub + (2 * c + 1) * 32 + r, (ss + 1) * 2 + hh);
+          } else {
+            fb[(ss + 1) & 1][2 * c - 4] = read_frag(slabQ, wm * kSub + (2 * c - 4) * 32 + r, (ss + 1) * 2 + hh);
+            fb[(ss + 1) & 1][2 * c - 3] = read_frag(slabQ, wm * kSub + (2 * c - 3) * 32 + r, (ss + 1) * 2 + hh);
+          }
         }
-      }
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma32(fa[ss & 1][nt], fb[ss & 1][mt], acc[nt][mt]);
-      // issue order: each LDS read of the NEXT sub-step's fragments is followed
-      // by two of this sub-step's MFMAs, so no MFMA waits on a read just issued
-      if (ss < 3) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 DS read
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // 2 MFMA
-        }
-      } else {
-        __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+        for (int mt = 0; mt < 4; ++mt) acc[c][mt] = mfma32(fa[ss & 1][c], fb[ss & 1][mt], acc[c][mt]);
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
     wait_vm0();
     __syncthreads();
   }
@@ -363,15 +369,27 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
   // pass 2: rescale each key block's partial sum and add the RBS rows of a query block
   const int kb_lo = lo / RBS, kb_hi = hi / RBS;
   float* out = p.sums + ((int64_t)head * p.nqb + mc / RBS) * p.nkb;
-  for (int kb = wave; kb < p.nkb; kb += 4) {
-    float w = 0.f;
-    if (real && kb >= kb_lo && kb <= kb_hi) {
-      const int T = (kb * RBS) / kSub;
-      w = Pst[(int64_t)kb * p.rows + mrel] * fast_exp2(Mst[(int64_t)T * p.rows + mrel] - safe) * inv;
+  // four independent key blocks per trip keep several loads in flight per lane
+  for (int kb0 = wave * 4; kb0 < p.nkb; kb0 += 16) {
+    float w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int kb = kb0 + u;
+      w[u] = 0.f;
+      if (real && kb >= kb_lo && kb <= kb_hi && kb < p.nkb) {
+        const int T = (kb * RBS) / kSub;
+        w[u] = Pst[(int64_t)kb * p.rows + mrel] * fast_exp2(Mst[(int64_t)T * p.rows + mrel] - safe) * inv;
+      }
     }
 #pragma unroll
-    for (int d = 1; d < RBS; d <<= 1) w += __shfl_xor(w, d, 64);
-    if (row_ok && (lane % RBS) == 0) out[kb] = w;
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int d = 1; d < RBS; d <<= 1) w[u] += __shfl_xor(w[u], d, 64);
+    if (row_ok && (lane % RBS) == 0) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (kb0 + u < p.nkb) out[kb0 + u] = w[u];
+    }
   }
 }
 
