@@ -75,3 +75,20 @@ def test_row_mass_invariant_large_logits():
     nb = L // 128
     upper = torch.triu(torch.ones(nb, nb, dtype=torch.bool), diagonal=1)
     assert (r["sums"].cpu()[:, upper] == 0).all()
+
+
+@pytest.mark.parametrize("is_causal", [True, False])
+def test_seam_flat_group_gemm_fuse_reshape(is_causal):
+    """The reference-named seam (xattn/src/kernels.py:325) on a middle query chunk."""
+    from xattn.src.kernels import flat_group_gemm_fuse_reshape, softmax_fuse_block_sum
+
+    S = 8
+    q, k = _mk(2, 2, 3 * S * 128, 3 * S * 128, 21)
+    qc = q[:, :, S * 128 : 2 * S * 128]            # second chunk of three
+    out = flat_group_gemm_fuse_reshape(qc.cuda(), k.cuda(), S, 128, 256, is_causal=is_causal)
+    want = O.antidiagonal_scores(qc.float(), k.float(), S)
+    assert out.shape == (1, 2, 128, 384) and out.dtype == torch.bfloat16
+    cols = 256 if is_causal else 384            # tiles past the chunk's diagonal are not computed
+    assert torch.allclose(out[..., :cols].float().cpu(), want[..., :cols], rtol=1e-2, atol=0.2)
+    with pytest.raises(NotImplementedError):
+        softmax_fuse_block_sum(out, 16, 16, 128, 256, 384, 1.0)

@@ -142,3 +142,23 @@ def test_operator_mask_and_output_parity(name, L, H, Hkv, S, C, tau, causal, use
     assert full.shape == (1, H, L, 128) and torch.isfinite(full.float()).all()
     if nbad == 0:
         assert (full.float().cpu() - want.float()).abs().max().item() <= OUT_MAX_ABS
+
+
+def test_seam_find_blocks_chunked_matches_reference_goldens():
+    """The reference-named seam (xattn/src/utils.py:44) against the golden masks,
+    cropped to each row's diagonal as the seam documents."""
+    from xattn.src.utils import find_blocks_chunked
+
+    for c in torch.load(GOLD, weights_only=True):
+        if c["name"] == "causal_dense_future":
+            continue
+        tau = c["threshold"] if c["threshold_is_tensor"] else float(c["threshold"])
+        got = find_blocks_chunked(c["x"].cuda(), c["current_index"], tau, None, decoding=False, mode="prefill", causal=c["causal"])
+        want = c["mask"].clone()
+        rows, cols = want.shape[2:]
+        if c["causal"]:
+            want &= torch.arange(cols)[None, :] <= torch.arange(rows)[:, None] + c["current_index"]
+        nbad, outside = mask_mismatch_report(c["x"][0].float(), got[0], want[0], tau, c["causal"], c["current_index"])
+        assert got.dtype == torch.bool and outside == 0, c["name"]
+    ones = find_blocks_chunked(torch.rand(1, 2, 4, 4).cuda(), 0, 0.9, None, decoding=True, mode="prefill")
+    assert ones.all()
