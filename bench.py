@@ -88,6 +88,8 @@ def main():
     ap.add_argument("--workload", type=int, default=2, help="index into the synthetic workloads (default: headline)")
     ap.add_argument("--dense-steps", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--compare-pipelined", action="store_true",
+                    help="also time Xattention_prefill with and without chunk-by-chunk stream pipelining")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) so that HBM byte "
                          "counters collected over this command can be scaled by a kernel of known traffic")
@@ -208,6 +210,22 @@ def main():
         },
     }
     del dense, out
+    if args.compare_pipelined:
+        from xattn.src.Xattention import Xattention_prefill
+
+        for flag in (False, True):
+            for _ in range(2):
+                Xattention_prefill(q, k, v, w.stride, threshold=w.threshold, chunk_size=chunk, causal=w.causal,
+                                   pipeline_chunks=flag)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                Xattention_prefill(q, k, v, w.stride, threshold=w.threshold, chunk_size=chunk, causal=w.causal,
+                                   pipeline_chunks=flag)
+            e1.record()
+            torch.cuda.synchronize()
+            result["operator_ms_pipelined" if flag else "operator_ms_single_launch"] = round(_ms(e0, e1) / args.steps, 3)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)

@@ -132,7 +132,9 @@ int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uin
  * idx_pitch entries long, as xattn_select_blocks writes them); inside a block, when causal, key c is visible to query t
  * iff c <= t + (k_len - q_len).  A query row with no visible key yields zeros.
  * col_idx == col_cnt == null visits every visible block: dense FlashAttention,
- * the baseline the speedup is quoted against.
+ * the baseline the speedup is quoted against.  Only query blocks
+ * [q_block_begin, q_block_end) are computed (q_block_end < 0: up to the last),
+ * so query chunks can be launched as their block lists become available.
  */
 int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* out,
                            const int32_t* col_idx, const int32_t* col_cnt, int64_t idx_pitch,
@@ -140,8 +142,8 @@ int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* ou
                            int head_dim,
                            int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                            int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
-                           int64_t o_stride_h, int64_t o_stride_n, int causal, float softmax_scale,
-                           void* stream);
+                           int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,
+                           int causal, float softmax_scale, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Measurement aid, no counterpart in the reference: copies `bytes` (a multiple

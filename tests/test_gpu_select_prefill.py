@@ -140,6 +140,11 @@ def test_operator_mask_and_output_parity(name, L, H, Hkv, S, C, tau, causal, use
     # and the operator end to end (its own mask)
     full = Xattention_prefill(q.cuda(), k.cuda(), v.cuda(), S, threshold=tau, chunk_size=C, causal=causal, use_triton=use_triton)
     assert full.shape == (1, H, L, 128) and torch.isfinite(full.float()).all()
+    # chunk-by-chunk orchestration on side streams computes the same thing
+    piped = Xattention_prefill(q.cuda(), k.cuda(), v.cuda(), S, threshold=tau, chunk_size=C, causal=causal,
+                               use_triton=use_triton, pipeline_chunks=True)
+    torch.cuda.synchronize()
+    assert torch.equal(piped, full)
     if nbad == 0:
         assert (full.float().cpu() - want.float()).abs().max().item() <= OUT_MAX_ABS
 

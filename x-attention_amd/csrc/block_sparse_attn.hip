@@ -43,6 +43,7 @@ struct AttnParams {
   int64_t idx_pitch;
   int idx_rows;             // q-block rows per head in col_idx / col_cnt (>= nqb)
   int H, Hkv, Lq, Lk, nqb, nkb;
+  int qb_begin, qb_end;     // q-blocks handled by this launch
   int causal, kv_off;       // kv_off = Lk - Lq
   float scale_log2;         // softmax_scale * log2(e)
 };
@@ -101,8 +102,8 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     const int x = id & 7, s = id >> 3;
     head = s % p.H;
     const int from_end = (s / p.H) * 8 + x;
-    if (from_end >= p.nqb) return;
-    qb = p.nqb - 1 - from_end;
+    if (from_end >= p.qb_end - p.qb_begin) return;
+    qb = p.qb_end - 1 - from_end;
   }
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
@@ -332,8 +333,8 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
                                       int idx_rows, int num_heads, int num_kv_heads, int q_len, int k_len, int head_dim,
                                       int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                                       int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
-                                      int64_t o_stride_h, int64_t o_stride_n, int causal, float softmax_scale,
-                                      void* stream) {
+                                      int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,
+                                      int causal, float softmax_scale, void* stream) {
   if (!q || !k || !v || !out) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
@@ -362,7 +363,11 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   if (col_idx && (idx_pitch < 1 || idx_rows < p.nqb)) return XATTN_ERR_SHAPE;
   p.idx_rows = idx_rows;
 
-  const int64_t grid = (int64_t)p.H * ((p.nqb + 7) / 8) * 8;
+  if (q_block_end < 0) q_block_end = p.nqb;
+  if (q_block_begin < 0 || q_block_begin >= q_block_end || q_block_end > p.nqb) return XATTN_ERR_SHAPE;
+  p.qb_begin = q_block_begin;
+  p.qb_end = q_block_end;
+  const int64_t grid = (int64_t)p.H * ((q_block_end - q_block_begin + 7) / 8) * 8;
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
   if (col_idx)
     hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(256), 0,

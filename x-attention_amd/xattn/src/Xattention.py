@@ -73,6 +73,90 @@ def _tau_per_head(threshold, heads, device):
     return torch.full((heads,), float(threshold), dtype=torch.float64, device=device)
 
 
+class _Plan:
+    """Geometry, buffers and kernel launchers of one estimate -> select pass."""
+
+    def __init__(self, query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores):
+        self.lib = _hb.lib()
+        q = _check_qk(query_states, "query_states")
+        k = _check_qk(key_states, "key_states")
+        if k.device != q.device:
+            k = k.to(q.device)
+        self.q, self.k = q, k
+        self.heads, self.q_len = q.shape[1], q.shape[2]
+        self.kv_heads, self.k_len = k.shape[1], k.shape[2]
+        if block_size != BLOCK:
+            raise AssertionError("block_size must be 128")
+        if stride not in (4, 8, 16):
+            raise ValueError("stride must be 4, 8 or 16")
+        if self.heads % self.kv_heads:
+            raise AssertionError("query heads must be a multiple of key/value heads")
+        if chunk_size % block_size:
+            raise AssertionError("chunk_size must be a multiple of block_size")
+        self.stride, self.chunk_size, self.block_size = stride, chunk_size, block_size
+        self.causal, self.keep_sink, self.keep_recent = bool(causal), bool(keep_sink), bool(keep_recent)
+        dev = self.dev = q.device
+        q_pad = -self.q_len % chunk_size
+        k_pad = -self.k_len % chunk_size
+        self.q_chunks = (self.q_len + q_pad) // chunk_size
+        assert (self.k_len + k_pad) // chunk_size >= self.q_chunks
+        self.nqb, self.nkb = (self.q_len + q_pad) // block_size, (self.k_len + k_pad) // block_size
+        self.blocks_per_chunk = chunk_size // block_size
+        self.own_chunk_only = self.causal and (not use_triton) and k_pad == 0
+        self.scale = 1.0 / math.sqrt(128) / stride / norm
+        self.list_cols = (self.k_len + block_size - 1) // block_size
+        self.ws_bytes = self.lib.xattn_estimate_workspace_bytes(
+            self.heads, self.q_len, self.k_len, stride, block_size, chunk_size, 0)
+        if self.ws_bytes == 0:
+            raise _hb.XattnHipError("estimator rejected the problem geometry")
+        with torch.cuda.device(dev):
+            self.workspace = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+            self.sums = torch.empty((self.heads, self.nqb, self.nkb), dtype=torch.float32, device=dev)
+            self.scores = None
+            if dump_scores:
+                self.scores = torch.zeros(
+                    (self.heads, (self.q_len + q_pad) // stride, (self.k_len + k_pad) // stride),
+                    dtype=torch.float32, device=dev)
+            self.tau = _tau_per_head(threshold, self.heads, dev)
+            self.mask = torch.empty((self.heads, self.nqb, self.nkb), dtype=torch.uint8, device=dev)
+            self.col_idx = self.col_cnt = None
+            if want_lists:
+                self.col_idx = torch.empty((self.heads, self.nqb, self.list_cols), dtype=torch.int32, device=dev)
+                self.col_cnt = torch.empty((self.heads, self.nqb), dtype=torch.int32, device=dev)
+
+    def estimate(self, chunk_begin, chunk_end, stream):
+        q, k = self.q, self.k
+        _hb.check(
+            self.lib.xattn_estimate_block_sums(
+                q.data_ptr(), k.data_ptr(), self.sums.data_ptr(), self.workspace.data_ptr(), self.ws_bytes,
+                self.scores.data_ptr() if self.scores is not None else None,
+                self.heads, self.kv_heads, self.q_len, self.k_len, 128,
+                q.stride(1), q.stride(2), k.stride(1), k.stride(2),
+                self.stride, self.block_size, self.chunk_size, chunk_begin, chunk_end,
+                int(self.causal), int(self.own_chunk_only), self.scale, stream,
+            ),
+            "xattn_estimate_block_sums",
+        )
+
+    def select(self, row_begin, row_end, stream):
+        lists = self.col_idx is not None
+        _hb.check(
+            self.lib.xattn_select_blocks(
+                self.sums.data_ptr(), self.tau.data_ptr(), self.mask.data_ptr(),
+                self.col_idx.data_ptr() if lists else None, self.col_cnt.data_ptr() if lists else None,
+                self.list_cols, self.heads, self.nqb, self.nkb, row_begin, row_end, self.nkb - self.nqb,
+                int(self.causal), int(self.keep_sink), int(self.keep_recent),
+                self.list_cols, self.q_len, self.k_len - self.q_len, self.blocks_per_chunk, stream,
+            ),
+            "xattn_select_blocks",
+        )
+
+    def result(self):
+        return dict(sums=self.sums, mask=self.mask, col_idx=self.col_idx, col_cnt=self.col_cnt,
+                    scores=self.scores, tau=self.tau)
+
+
 def estimate_and_select(
     query_states,
     key_states,
@@ -89,86 +173,26 @@ def estimate_and_select(
     dump_scores=False,
     marks=None,
 ):
-    """Runs the estimator and selection kernels.
-
-    ``marks``, when a list, receives ``(label, torch.cuda.Event)`` pairs recorded
-    on the current stream before the estimator, between estimator and selection
-    and after selection (for per-kernel timing).
+    """Runs the estimator and selection kernels over all query chunks, one launch each.
 
     Returns a dict with fp32 ``sums`` [H, Nq_p, Nk_p], uint8 ``mask`` of the same
     shape, and (when ``want_lists``) ``col_idx`` [H, Nq_p, pitch] / ``col_cnt``
     [H, Nq_p] for :func:`block_sparse_attention`.
-    """
-    lib = _hb.lib()
-    q = _check_qk(query_states, "query_states")
-    k = _check_qk(key_states, "key_states")
-    if k.device != q.device:
-        k = k.to(q.device)
-    heads, q_len = q.shape[1], q.shape[2]
-    kv_heads, k_len = k.shape[1], k.shape[2]
-    if block_size != BLOCK:
-        raise AssertionError("block_size must be 128")
-    if stride not in (4, 8, 16):
-        raise ValueError("stride must be 4, 8 or 16")
-    if heads % kv_heads:
-        raise AssertionError("query heads must be a multiple of key/value heads")
-    if chunk_size % block_size:
-        raise AssertionError("chunk_size must be a multiple of block_size")
-    dev = q.device
-    q_pad = -q_len % chunk_size
-    k_pad = -k_len % chunk_size
-    q_chunks = (q_len + q_pad) // chunk_size
-    k_chunks = (k_len + k_pad) // chunk_size
-    assert k_chunks >= q_chunks
-    nqb, nkb = (q_len + q_pad) // block_size, (k_len + k_pad) // block_size
-    own_chunk_only = bool(causal) and (not use_triton) and k_pad == 0
 
-    with torch.cuda.device(dev):
-        stream = _stream_ptr(dev)
-        ws_bytes = lib.xattn_estimate_workspace_bytes(heads, q_len, k_len, stride, block_size, chunk_size, 0)
-        if ws_bytes == 0:
-            raise _hb.XattnHipError("estimator rejected the problem geometry")
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-        sums = torch.empty((heads, nqb, nkb), dtype=torch.float32, device=dev)
-        scores = None
-        if dump_scores:
-            scores = torch.zeros(
-                (heads, (q_len + q_pad) // stride, (k_len + k_pad) // stride), dtype=torch.float32, device=dev
-            )
-        scale = 1.0 / math.sqrt(128) / stride / norm
+    ``marks``, when a list, receives ``(label, torch.cuda.Event)`` pairs recorded
+    on the current stream before the estimator, between estimator and selection
+    and after selection (for per-kernel timing).
+    """
+    plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores)
+    with torch.cuda.device(plan.dev):
+        stream = _stream_ptr(plan.dev)
         _mark(marks, "estimate_begin")
-        _hb.check(
-            lib.xattn_estimate_block_sums(
-                q.data_ptr(), k.data_ptr(), sums.data_ptr(), workspace.data_ptr(), ws_bytes,
-                scores.data_ptr() if scores is not None else None,
-                heads, kv_heads, q_len, k_len, 128,
-                q.stride(1), q.stride(2), k.stride(1), k.stride(2),
-                stride, block_size, chunk_size, 0, q_chunks, int(bool(causal)), int(own_chunk_only),
-                scale, stream,
-            ),
-            "xattn_estimate_block_sums",
-        )
-        tau = _tau_per_head(threshold, heads, dev)
+        plan.estimate(0, plan.q_chunks, stream)
         _mark(marks, "select_begin")
-        mask = torch.empty((heads, nqb, nkb), dtype=torch.uint8, device=dev)
-        col_idx = col_cnt = None
-        list_cols = (k_len + block_size - 1) // block_size
-        if want_lists:
-            col_idx = torch.empty((heads, nqb, list_cols), dtype=torch.int32, device=dev)
-            col_cnt = torch.empty((heads, nqb), dtype=torch.int32, device=dev)
-        _hb.check(
-            lib.xattn_select_blocks(
-                sums.data_ptr(), tau.data_ptr(), mask.data_ptr(),
-                col_idx.data_ptr() if want_lists else None,
-                col_cnt.data_ptr() if want_lists else None,
-                list_cols, heads, nqb, nkb, 0, nqb, nkb - nqb,
-                int(bool(causal)), int(bool(keep_sink)), int(bool(keep_recent)),
-                list_cols, q_len, k_len - q_len, chunk_size // block_size, stream,
-            ),
-            "xattn_select_blocks",
-        )
+        plan.select(0, plan.nqb, stream)
         _mark(marks, "select_end")
-    return dict(sums=sums, mask=mask, col_idx=col_idx, col_cnt=col_cnt, scores=scores, tau=tau)
+    return plan.result()
 
 
 def xattn_estimate(
@@ -212,12 +236,14 @@ def xattn_estimate(
 
 
 def block_sparse_attention(query_states, key_states, value_states, col_idx=None, col_cnt=None,
-                           causal=True, softmax_scale=None):
+                           causal=True, softmax_scale=None, out=None, q_blocks=None, stream=None):
     """Attention of each 128-token query block over the key blocks listed for it
     (``col_idx``/``col_cnt`` as written by :func:`estimate_and_select`; ``None``
     visits every visible block = dense FlashAttention).  Stands in for
     ``block_sparse_attn_func`` at xattn/src/Xattention.py:377-391.
     Returns ``[1, H, q_len, 128]`` as a transposed view of ``[1, q_len, H, 128]``.
+    ``out`` (a ``[1, q_len, H, 128]`` buffer), ``q_blocks=(begin, end)`` and ``stream``
+    (a ``torch.cuda.Stream``) let a caller fill the output chunk by chunk.
     """
     lib = _hb.lib()
     q = _check_qk(query_states, "query_states")
@@ -234,7 +260,9 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
         raise AssertionError("key_states and value_states must agree in heads and length")
     if (col_idx is None) != (col_cnt is None):
         raise AssertionError("col_idx and col_cnt go together")
-    out = torch.empty((1, q_len, heads, 128), dtype=torch.bfloat16, device=dev)
+    if out is None:
+        out = torch.empty((1, q_len, heads, 128), dtype=torch.bfloat16, device=dev)
+    qb0, qb1 = q_blocks if q_blocks is not None else (0, -1)
     scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(128)
     if col_idx is not None:
         assert col_idx.dtype == torch.int32 and col_cnt.dtype == torch.int32
@@ -251,7 +279,8 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
                 col_cnt.data_ptr() if col_cnt is not None else None,
                 pitch, idx_rows, heads, kv_heads, q_len, k_len, 128,
                 q.stride(1), q.stride(2), k.stride(1), k.stride(2), v.stride(1), v.stride(2),
-                out.stride(2), out.stride(1), int(bool(causal)), scale, _stream_ptr(dev),
+                out.stride(2), out.stride(1), qb0, qb1, int(bool(causal)), scale,
+                stream.cuda_stream if stream is not None else _stream_ptr(dev),
             ),
             "xattn_block_sparse_fwd",
         )
@@ -272,10 +301,13 @@ def Xattention_prefill(
     chunk_size=None,
     keep_sink=False,
     keep_recent=False,
+    pipeline_chunks=False,
 ):
     """Sparse prefill attention: antidiagonal estimate -> block selection ->
     block-sparse FlashAttention.  Signature, defaults and result layout of
-    xattn/src/Xattention.py:302-402."""
+    xattn/src/Xattention.py:302-402.  ``pipeline_chunks=True`` (not in the
+    reference) issues the three stages query chunk by query chunk on separate HIP
+    streams instead of one launch per stage; the result is the same."""
     batch_size, _, k_len, _ = key_states.shape
     assert block_size == 128
     assert batch_size == 1
@@ -283,6 +315,9 @@ def Xattention_prefill(
         raise ValueError("kdb != 1 is not supported by the fused estimator")
     if chunk_size is None:
         chunk_size = default_chunk_size(k_len)
+    if pipeline_chunks:
+        return _prefill_pipelined(query_states, key_states, value_states, stride, norm, threshold, block_size,
+                                  use_triton, causal, chunk_size, keep_sink, keep_recent)
     r = estimate_and_select(
         query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
         use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
@@ -291,3 +326,62 @@ def Xattention_prefill(
     return block_sparse_attention(
         query_states, key_states, value_states, r["col_idx"], r["col_cnt"], causal=causal
     )
+
+
+_side_streams = {}
+
+
+def _streams(dev):
+    """Two side streams per device, default priority, created once."""
+    key = (dev.type, dev.index)
+    if key not in _side_streams:
+        _side_streams[key] = (torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev))
+    return _side_streams[key]
+
+
+def _prefill_pipelined(query_states, key_states, value_states, stride, norm, threshold, block_size, use_triton,
+                       causal, chunk_size, keep_sink, keep_recent):
+    """Chunk-by-chunk orchestration on three HIP streams: the estimator of query
+    chunk c runs on the caller's stream, the selection of chunk c on a second
+    stream as soon as its block sums exist, and the attention of chunk c's query
+    blocks on a third as soon as its column lists exist - so selection and
+    attention of earlier chunks fill the compute units the estimator's tail
+    leaves idle.  The caller's stream waits for both side streams before the
+    function returns, which also makes every temporary safe to free."""
+    plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
+                 keep_sink, keep_recent, block_size, True, False)
+    dev = plan.dev
+    q = plan.q
+    k = plan.k
+    v = _check_qk(value_states, "value_states")
+    if v.device != dev:
+        v = v.to(dev)
+    nb = (plan.q_len + block_size - 1) // block_size
+    with torch.cuda.device(dev):
+        main = torch.cuda.current_stream(dev)
+        s_sel, s_att = _streams(dev)
+        out = torch.empty((1, plan.q_len, plan.heads, 128), dtype=torch.bfloat16, device=dev)
+        start = torch.cuda.Event()
+        start.record(main)
+        s_sel.wait_event(start)
+        s_att.wait_event(start)
+        bpc = plan.blocks_per_chunk
+        for c in range(plan.q_chunks):
+            plan.estimate(c, c + 1, main.cuda_stream)
+            ev = torch.cuda.Event()
+            ev.record(main)
+            s_sel.wait_event(ev)
+            plan.select(c * bpc, (c + 1) * bpc, s_sel.cuda_stream)
+            ev2 = torch.cuda.Event()
+            ev2.record(s_sel)
+            qb0, qb1 = c * bpc, min(nb, (c + 1) * bpc)
+            if qb0 < qb1:
+                s_att.wait_event(ev2)
+                block_sparse_attention(q, k, v, plan.col_idx, plan.col_cnt, causal=causal, out=out,
+                                       q_blocks=(qb0, qb1), stream=s_att)
+        done_sel, done_att = torch.cuda.Event(), torch.cuda.Event()
+        done_sel.record(s_sel)
+        done_att.record(s_att)
+        main.wait_event(done_sel)
+        main.wait_event(done_att)
+    return out.transpose(1, 2)
