@@ -172,60 +172,78 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
+  // k-step t covers token i = t / 2 of every reshaped row's group, features
+  // 64*(t % 2) .. +63, and is read from LDS stage t % 2.
+  //
+  // Software pipeline.  A step is four sub-steps of 16 MFMAs; the 8 fragment
+  // reads of the next sub-step and 4 of the 16 copies of a later step are
+  // issued between them, in chunks the scheduler may not mix (one copy, two
+  // reads, four MFMAs: with one wavefront per SIMD issue is in order, so a burst
+  // of copies or reads would hold back the MFMAs queued behind it).  The
+  // workgroup barrier sits before the LAST sub-step's MFMAs: at that point every
+  // fragment of the current stage has been read, so the sub-step can prefetch
+  // the next stage's first fragments and start refilling the current stage
+  // while its MFMAs run - the MFMA stream never drains at a step boundary.
   const int steps = p.S * 2;
   int voffK[8], voffQ[8];
   slab_offsets(k_snb, n0, p.S, lane, wave, voffK);
   slab_offsets(q_snb, m0, p.S, lane, wave, voffQ);
-  copy_slab(kres, voffK, 0, lds, wave);
-  copy_slab(qres, voffQ, (p.S - 1) * (int)q_snb, lds + kTile * 128, wave);
+  auto step_off_k = [&](int t) { return (t >> 1) * (int)k_snb + (t & 1) * kDepth * 2; };
+  auto step_off_q = [&](int t) { return (p.S - 1 - (t >> 1)) * (int)q_snb + (t & 1) * kDepth * 2; };
+  // copy j (0..15) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
+  auto copy_j = [&](int j, int t, char* stage) {
+    const int tc = t < steps ? t : steps - 1;       // past the end: a harmless repeat
+    if (j & 1) copy_one(qres, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
+    else copy_one(kres, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
+  };
+#pragma unroll
+  for (int j = 0; j < 16; ++j) copy_j(j, 0, lds);
   wait_vm0();
   __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) copy_j(j, 1, lds + kStageBytes);
+
+  bf16x8 fa[2][4], fb[2][4];
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    fa[0][x] = read_frag(lds, wn * kSub + x * 32 + r, hh);
+    fb[0][x] = read_frag(lds + kTile * 128, wm * kSub + x * 32 + r, hh);
+  }
 
   for (int t = 0; t < steps; ++t) {
     char* cur = lds + (t & 1) * kStageBytes;
     char* nxt = lds + ((t + 1) & 1) * kStageBytes;
-    // the last step copies its own slabs again into the idle stage, which keeps
-    // the loop body free of branches
-    const int tn = t + 1 < steps ? t + 1 : t;
-    const int offK = (tn >> 1) * (int)k_snb + (tn & 1) * kDepth * 2;
-    const int offQ = (p.S - 1 - (tn >> 1)) * (int)q_snb + (tn & 1) * kDepth * 2;
-    const char* slabK = cur;
-    const char* slabQ = cur + kTile * 128;
-    bf16x8 fa[2][4], fb[2][4];
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      fa[0][x] = read_frag(slabK, wn * kSub + x * 32 + r, hh);
-      fb[0][x] = read_frag(slabQ, wm * kSub + x * 32 + r, hh);
-    }
-    // The step is cut into 16 chunks that the scheduler may not mix: one of the
-    // 16 copies of the next k-step, two of the 8 fragment reads of the next
-    // sub-step, four MFMAs.  With one wavefront per SIMD issue is in order, so a
-    // burst of copies or reads would hold back the MFMAs queued behind it.
 #pragma unroll
     for (int ss = 0; ss < 4; ++ss) {
+      if (ss == 3) {
+        // every copy of step t+1 has landed; every wavefront has read its last
+        // fragment of step t (the reads were issued during sub-step 2)
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vm0();
+        __syncthreads();
+      }
+      const char* fragK = ss < 3 ? cur : nxt;             // where the next sub-step's fragments live
+      const char* fragQ = fragK + kTile * 128;
+      const int nss = (ss + 1) & 3;                        // its sub-step index within that stage
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         __builtin_amdgcn_sched_barrier(0);
-        const int it = ss * 2 + (c >> 1);
-        if (c & 1) copy_one(qres, voffQ[it], offQ, nxt + kTile * 128, wave, it);
-        else copy_one(kres, voffK[it], offK, nxt, wave, it);
-        if (ss < 3) {
-          if (c < 2) {
-            fa[(ss + 1) & 1][2 * c] = read_frag(slabK, wn * kSub + (2 * c) * 32 + r, (ss + 1) * 2 + hh);
-            fa[(ss + 1) & 1][2 * c + 1] = read_frag(slabK, wn * kSub + (2 * c + 1) * 32 + r, (ss + 1) * 2 + hh);
-          } else {
-            fb[(ss + 1) & 1][2 * c - 4] = read_frag(slabQ, wm * kSub + (2 * c - 4) * 32 + r, (ss + 1) * 2 + hh);
-            fb[(ss + 1) & 1][2 * c - 3] = read_frag(slabQ, wm * kSub + (2 * c - 3) * 32 + r, (ss + 1) * 2 + hh);
-          }
+        if (ss < 3) copy_j(4 + ss * 4 + c, t + 1, nxt);    // copies 4..15 of step t+1
+        else copy_j(c, t + 2, cur);                        // copies 0..3 of step t+2 refill this stage
+        if (c < 2) {
+          fa[(ss + 1) & 1][2 * c] = read_frag(fragK, wn * kSub + (2 * c) * 32 + r, nss * 2 + hh);
+          fa[(ss + 1) & 1][2 * c + 1] = read_frag(fragK, wn * kSub + (2 * c + 1) * 32 + r, nss * 2 + hh);
+        } else {
+          fb[(ss + 1) & 1][2 * c - 4] = read_frag(fragQ, wm * kSub + (2 * c - 4) * 32 + r, nss * 2 + hh);
+          fb[(ss + 1) & 1][2 * c - 3] = read_frag(fragQ, wm * kSub + (2 * c - 3) * 32 + r, nss * 2 + hh);
         }
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) acc[c][mt] = mfma32(fa[ss & 1][c], fb[ss & 1][mt], acc[c][mt]);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    wait_vm0();
-    __syncthreads();
   }
+  wait_vm0();   // the repeats issued by the last steps
 
   // ---- epilogue: this wavefront's 128 keys x 128 query rows
   const int nbase = n0 + wn * kSub;       // first key of the wavefront tile
