@@ -237,11 +237,24 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
       for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[nt][v]);
-    mx = fmaxf(mx, swap_half(mx));
-    const float m_new = fmaxf(m_run, mx * p.scale_log2);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_safe);
-    m_run = m_new;
+    mx = fmaxf(mx, swap_half(mx)) * p.scale_log2;
+    // The reference maximum m_run is only moved when a row's maximum outgrows it
+    // by more than 2^8 (or on the row's first visible key): exp2 arguments then
+    // stay <= 8, which fp32 sums and bf16 probabilities hold without loss, and
+    // the rescaling of l and of the 64 output accumulators is skipped for the
+    // wavefront whenever no row needs it.  O / l does not depend on the choice.
+    const bool move = mx > m_run + 8.f || (m_run == -INFINITY && mx > -INFINITY);
+    if (__any(move)) {
+      const float m_new = move ? mx : m_run;
+      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+    }
+    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
     float psum = 0.f;
     bf16x8 pfrag[8];
 #pragma unroll
@@ -252,11 +265,7 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
         psum += e;
         pfrag[nt * 2 + (v >> 3)][v & 7] = (__bf16)e;
       }
-    l_run = l_run * alpha + psum;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+    l_run += psum;
 
     // ---- O^T += V_j^T P^T
     {
