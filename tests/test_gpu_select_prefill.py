@@ -167,3 +167,25 @@ def test_seam_find_blocks_chunked_matches_reference_goldens():
         assert got.dtype == torch.bool and outside == 0, c["name"]
     ones = find_blocks_chunked(torch.rand(1, 2, 4, 4).cuda(), 0, 0.9, None, decoding=True, mode="prefill")
     assert ones.all()
+
+
+def test_operator_with_kv_longer_than_q():
+    """Chunked prefill against a KV cache (k_len > q_len): the block diagonal and the
+    token-causal mask are bottom-right aligned (xattn/src/Xattention.py:39-40, 153-157, 257)."""
+    from xattn.src.Xattention import Xattention_prefill, xattn_estimate
+    from xattn.synthetic import WORKLOADS, make_inputs
+
+    S, C, Lq, Lk, H, Hkv = 8, 2048, 2048, 6144, 8, 2
+    q_all, k, v = make_inputs(WORKLOADS[1], device="cpu", seed=11, L=Lk, heads=H, kv_heads=Hkv)
+    q = q_all[:, :, -Lq:].contiguous()
+    kf, vf = k.repeat_interleave(H // Hkv, 1).float(), v.repeat_interleave(H // Hkv, 1).float()
+    want_sums, want_mask = O.xattn_estimate(q.float(), kf, 128, S, threshold=0.9, chunk_size=C, pad0_quirk=False)
+    sums, mask = xattn_estimate(q.cuda(), k.cuda(), 128, S, threshold=0.9, chunk_size=C)
+    assert mask.shape == (1, H, Lq // 128, Lk // 128)
+    nbad, outside = mask_mismatch_report(want_sums[0], mask[0], want_mask[0], 0.9, True, (Lk - Lq) // 128, C // 128)
+    assert outside == 0 and nbad <= 2
+    want = O.block_sparse_attention(q, k, v, want_mask, causal=True)
+    out = Xattention_prefill(q.cuda(), k.cuda(), v.cuda(), S, threshold=0.9, chunk_size=C)
+    if nbad == 0:
+        err = (out.float().cpu() - want.float()).abs()
+        assert err.max().item() <= OUT_MAX_ABS and err.mean().item() <= OUT_MEAN_ABS

@@ -32,7 +32,6 @@ struct EstParams {
   const __bf16* q;
   const __bf16* k;
   int64_t q_sh, q_sn, k_sh, k_sn;
-  int64_t q_bytes, k_bytes;   // per-head extent q_len * q_sn * 2 (tokens beyond read as zeros)
   float* P;        // [H][nkb][rows]  partial block sums relative to the tile maximum
   float* Mt;       // [H][nT][rows]   tile maximum (exp2 domain)
   float* Lt;       // [H][nT][rows]   tile sum
@@ -73,18 +72,15 @@ __device__ __forceinline__ int row_hi(const EstParams& p, int m) {
 // position c fetches chunk c ^ ((r >> 1) & 7)).
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-// Per-lane byte offsets of the 8 rows a lane copies per slab, for token 0 of
-// each reshaped row's group and feature 0; the k-step adds a uniform term.
-// Offsets that do not fit 31 bits are pinned there: the host guarantees every
-// valid byte lies below 2^31, so they (and anything they grow into) read zeros.
-__device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int first_row, int S, int lane, int wave,
-                                             int (&voff)[8]) {
+// Per-lane byte offsets (relative to the tile's first token) of the 8 rows a
+// lane copies per slab, for token 0 of each reshaped row's group and feature 0;
+// the k-step adds a uniform term.  The host checks that a tile spans < 2^31 bytes.
+__device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int S, int lane, int wave, int (&voff)[8]) {
   const int c = lane & 7, rl = lane >> 3;
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int r = it * 32 + wave * 8 + rl;
-    const int64_t off = (int64_t)(first_row + r) * S * sn_bytes + ((c ^ ((r >> 1) & 7)) << 4);
-    voff[it] = off < 0x7fffffff ? (int)off : 0x7fffffff;
+    voff[it] = (int)((int64_t)r * S * sn_bytes) + ((c ^ ((r >> 1) & 7)) << 4);
   }
 }
 
@@ -158,11 +154,19 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
-  const __amdgpu_buffer_rsrc_t qres =
-      __builtin_amdgcn_make_buffer_rsrc((void*)qbase, 0, (int)p.q_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t kres =
-      __builtin_amdgcn_make_buffer_rsrc((void*)kbase, 0, (int)p.k_bytes, 0x00020000);
+  // Buffer resources are rebased to the tile's first token and end at the real
+  // sequence end (or the tile's end), so lane offsets stay small whatever the
+  // token stride, and tokens past the real length read as zeros.
   const int64_t q_snb = p.q_sn * 2, k_snb = p.k_sn * 2;
+  const int64_t q_tok0 = (int64_t)m0 * p.S, k_tok0 = (int64_t)n0 * p.S;
+  const int64_t q_left = p.Lq - q_tok0, k_left = p.Lk - k_tok0;
+  const int64_t span = (int64_t)kTile * p.S;
+  const int64_t q_rows = q_left < 0 ? 0 : (q_left < span ? q_left : span);
+  const int64_t k_rows = k_left < 0 ? 0 : (k_left < span ? k_left : span);
+  const __amdgpu_buffer_rsrc_t qres = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(qbase + (q_rows > 0 ? q_tok0 * p.q_sn : 0)), 0, (int)(q_rows * q_snb), 0x00020000);
+  const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(kbase + (k_rows > 0 ? k_tok0 * p.k_sn : 0)), 0, (int)(k_rows * k_snb), 0x00020000);
 
   f32x16 acc[4][4];   // [key tile nt][query tile mt]
 #pragma unroll
@@ -186,8 +190,8 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   // while its MFMAs run - the MFMA stream never drains at a step boundary.
   const int steps = p.S * 2;
   int voffK[8], voffQ[8];
-  slab_offsets(k_snb, n0, p.S, lane, wave, voffK);
-  slab_offsets(q_snb, m0, p.S, lane, wave, voffQ);
+  slab_offsets(k_snb, p.S, lane, wave, voffK);
+  slab_offsets(q_snb, p.S, lane, wave, voffQ);
   auto step_off_k = [&](int t) { return (t >> 1) * (int)k_snb + (t & 1) * kDepth * 2; };
   auto step_off_q = [&](int t) { return (p.S - 1 - (t >> 1)) * (int)q_snb + (t & 1) * kDepth * 2; };
   // copy j (0..15) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
@@ -483,10 +487,11 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.q = static_cast<const __bf16*>(q);
   p.k = static_cast<const __bf16*>(k);
   p.q_sh = q_stride_h; p.q_sn = q_stride_n; p.k_sh = k_stride_h; p.k_sn = k_stride_n;
-  p.q_bytes = (int64_t)q_len * q_stride_n * 2;
-  p.k_bytes = (int64_t)k_len * k_stride_n * 2;
   if (q_stride_n < kHeadDim || k_stride_n < kHeadDim) return XATTN_ERR_ALIGN;
-  if (p.q_bytes >= 0x7fffffff || p.k_bytes >= 0x7fffffff) return XATTN_ERR_SHAPE;
+  // one 256-row tile (256 * stride tokens) must span less than 2^31 bytes
+  if ((int64_t)(kTile + 1) * stride * q_stride_n * 2 >= 0x7fffffff ||
+      (int64_t)(kTile + 1) * stride * k_stride_n * 2 >= 0x7fffffff)
+    return XATTN_ERR_SHAPE;
   p.H = num_heads; p.Hkv = num_kv_heads; p.Lq = q_len; p.Lk = k_len; p.S = stride;
   p.rbs = block_size / stride;
   p.n_rq = g.n_rq; p.n_rk = g.n_rk; p.nkb = g.nkb; p.nqb = g.nqb; p.nT = g.nT; p.rcs = g.rcs;
