@@ -61,6 +61,16 @@ def cpu_baseline(reps=5, warmup=2):
                 t_est.append((t1 - t0) * 1e3)
                 t_att.append((t2 - t1) * 1e3)
     est, att = statistics.median(t_est), statistics.median(t_att)
+    with torch.no_grad():
+        # the other setting of the torch-branch slice quirk (keys of earlier chunks visible), for the record
+        _, mask_all_keys = O.xattn_estimate(q, k, 128, w.stride, threshold=w.threshold, chunk_size=w.chunk_size,
+                                            causal=True, pad0_quirk=False)
+        torch.set_num_threads(1)
+        t0 = time.perf_counter()
+        _, m1 = O.xattn_estimate(q, k, 128, w.stride, threshold=w.threshold, chunk_size=w.chunk_size, causal=True)
+        O.block_sparse_attention(q, k, v, m1, causal=True)
+        single = (time.perf_counter() - t0) * 1e3
+        torch.set_num_threads(threads)
     return {
         "value": round(est + att, 3),
         "unit": "ms per layer",
@@ -76,7 +86,9 @@ def cpu_baseline(reps=5, warmup=2):
         "torch_threads": torch.get_num_threads(),
         "os_cpu_count": cores,
         "torch": torch.__version__,
+        "single_thread_ms": round(single, 1),
         "mask_density": round(float(mask.float().mean()), 4),
+        "mask_density_all_earlier_keys_visible": round(float(mask_all_keys.float().mean()), 4),
     }, (q, k, v, mask)
 
 
@@ -254,7 +266,9 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         base["gpu_same_sample_ms"] = round(_ms(e0, e1) / 10, 3)
+        # (the GPU sees the sample rounded to bf16, the CPU oracle ran it in fp32: a few threshold-edge blocks differ)
         base["gpu_mask_mismatch_vs_cpu"] = int((rr["mask"].bool().cpu() != cmask[0]).sum())
+        base["gpu_mask_blocks"] = int(cmask[0].numel())
         result["cpu_baseline"] = base
     print(json.dumps(result))
 

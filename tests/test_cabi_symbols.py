@@ -65,3 +65,21 @@ def test_operator_refuses_cpu_tensors_and_wrong_dtypes():
     table = {1024: 2048, 4096: 4096, 16384: 16384, 32768: 8192, 65536: 4096, 131072: 2048, 119056: 2048}
     for L, want in table.items():
         assert default_chunk_size(L) == want
+
+
+def test_product_path_never_touches_the_oracle():
+    """The oracle is a checker: nothing under the package may import or run it."""
+    pkg = os.path.join(ROOT, "x-attention_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(base, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text and "xattn_oracle" not in text, f
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr
