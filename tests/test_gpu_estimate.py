@@ -92,3 +92,13 @@ def test_seam_flat_group_gemm_fuse_reshape(is_causal):
     assert torch.allclose(out[..., :cols].float().cpu(), want[..., :cols], rtol=1e-2, atol=0.2)
     with pytest.raises(NotImplementedError):
         softmax_fuse_block_sum(out, 16, 16, 128, 256, 384, 1.0)
+
+
+def test_workspace_limit_splits_the_launch_without_changing_results(monkeypatch):
+    import xattn.src.Xattention as X
+
+    q, k = _mk(4, 2, 4096, 4096, 33)
+    a = X.estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, causal=True, want_lists=False)["sums"].clone()
+    monkeypatch.setattr(X, "WORKSPACE_LIMIT", 1 << 20)     # forces several chunk groups
+    b = X.estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, causal=True, want_lists=False)["sums"]
+    assert torch.equal(a, b)

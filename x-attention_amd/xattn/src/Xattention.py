@@ -27,6 +27,7 @@ from . import hip_backend as _hb
 __all__ = ["Xattention_prefill", "xattn_estimate", "default_chunk_size", "estimate_and_select", "block_sparse_attention"]
 
 BLOCK = 128
+WORKSPACE_LIMIT = 4 << 30   # bytes of estimator workspace per launch
 
 
 def default_chunk_size(k_len):
@@ -106,10 +107,15 @@ class _Plan:
         self.own_chunk_only = self.causal and (not use_triton) and k_pad == 0
         self.scale = 1.0 / math.sqrt(128) / stride / norm
         self.list_cols = (self.k_len + block_size - 1) // block_size
-        self.ws_bytes = self.lib.xattn_estimate_workspace_bytes(
-            self.heads, self.q_len, self.k_len, stride, block_size, chunk_size, 0)
-        if self.ws_bytes == 0:
+        # The estimator's workspace grows with (query rows per call) x (key blocks); very long
+        # sequences are processed in groups of query chunks that keep it under WORKSPACE_LIMIT.
+        per_chunk = self.lib.xattn_estimate_workspace_bytes(
+            self.heads, self.q_len, self.k_len, stride, block_size, chunk_size, 1)
+        if per_chunk == 0:
             raise _hb.XattnHipError("estimator rejected the problem geometry")
+        self.chunks_per_call = max(1, min(self.q_chunks, WORKSPACE_LIMIT // per_chunk))
+        self.ws_bytes = self.lib.xattn_estimate_workspace_bytes(
+            self.heads, self.q_len, self.k_len, stride, block_size, chunk_size, self.chunks_per_call)
         with torch.cuda.device(dev):
             self.workspace = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
             self.sums = torch.empty((self.heads, self.nqb, self.nkb), dtype=torch.float32, device=dev)
@@ -126,6 +132,10 @@ class _Plan:
                 self.col_cnt = torch.empty((self.heads, self.nqb), dtype=torch.int32, device=dev)
 
     def estimate(self, chunk_begin, chunk_end, stream):
+        if chunk_end - chunk_begin > self.chunks_per_call:
+            for c in range(chunk_begin, chunk_end, self.chunks_per_call):
+                self.estimate(c, min(chunk_end, c + self.chunks_per_call), stream)
+            return
         q, k = self.q, self.k
         _hb.check(
             self.lib.xattn_estimate_block_sums(
