@@ -4,11 +4,16 @@
 // the mask post-processing of xattn_estimate (xattn/src/Xattention.py:275-297).
 // The reference runs ~15 eager torch ops over an fp64 copy of the block sums
 // (two full sorts, a cumsum, an advanced-index scatter) and synchronises the
-// device once per chunk; here a row's candidates are sorted by a bitonic
-// network in LDS (only the columns up to the diagonal when causal - a
-// "segmented" sort whose size follows the row), the fp64 prefix sum is a
-// wavefront scan, and the kernel emits the final mask row plus the compacted,
-// ascending column list the attention kernel walks.
+// device once per chunk; here a row's candidates (only the columns up to the
+// diagonal when causal - the problem size follows the row) are first tried by
+// extraction: the wavefront pulls out the largest remaining block, adds its
+// mass, and stops as soon as the threshold is reached - on sparse rows that is a
+// handful of wavefront reductions.  Rows that need more than kMaxExtract blocks
+// fall back to a bitonic sort of the candidates in LDS followed by an fp64
+// wavefront prefix scan.  Both visit blocks in the same order (descending sum,
+// ascending column among equals) and apply the same rule.  The kernel emits the
+// final mask row plus the compacted, ascending column list the attention kernel
+// walks.
 #include "xattn_common.h"
 #include "xattn_hip.h"
 
@@ -26,6 +31,9 @@ struct SelParams {
   int blocks_per_chunk;
   int npow2;   // LDS key capacity (power of two >= nkb)
 };
+
+constexpr int kSlots = 16;        // candidates per lane held in registers (rows up to 1024 candidates)
+constexpr int kMaxExtract = 32;   // blocks pulled out one by one before falling back to the sort
 
 // value encoded in a sort key (0 for forced blocks and padding)
 __device__ __forceinline__ double key_value(uint64_t key) {
@@ -67,8 +75,13 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   while (np2 < ncand) np2 <<= 1;
 
   double total = 0.0;
-  for (int c = lane; c < np2; c += 64) {
+  uint32_t vals[kSlots];      // this lane's candidates: slot u holds column u*64 + lane (0 = none)
+  int n_others = 0;
+#pragma unroll
+  for (int u = 0; u < kSlots; ++u) vals[u] = 0;
+  auto load_one = [&](int c) -> uint32_t {
     uint64_t key = 0;   // padding sorts last and carries an out-of-range column
+    uint32_t bits = 0;
     if (c < ncand) {
       const float v = x[c];
       total += (double)v;
@@ -76,10 +89,22 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
       // block sums are >= 0, so their bit pattern orders like the value (+1
       // keeps every candidate ahead of the forced blocks, which sort last);
       // low word = ~column makes equal sums come out by ascending column
-      const uint32_t bits = forced ? 0u : __float_as_uint(v > 0.f ? v : 0.f) + 1u;
+      bits = forced ? 0u : __float_as_uint(v > 0.f ? v : 0.f) + 1u;
       key = ((uint64_t)bits << 32) | (uint32_t)(~(uint32_t)c);
     }
     keys[c] = key;
+    return bits;
+  };
+  const bool small = np2 <= kSlots * 64;
+  if (small) {
+#pragma unroll
+    for (int u = 0; u < kSlots; ++u)
+      if (u * 64 < np2) {
+        vals[u] = load_one(u * 64 + lane);
+        n_others += vals[u] != 0;
+      }
+  } else {
+    for (int c = lane; c < np2; c += 64) load_one(c);
   }
   for (int c = lane; c < p.nkb; c += 64) flags[c] = 0;
   total = wave_sum(total);
@@ -91,7 +116,47 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   }
   __syncthreads();
 
-  // bitonic sort, descending
+  int dropped = 0;
+  bool finished = false;
+  if (small) {
+    // ---- extraction: keep pulling out the largest remaining block while the rule says "keep"
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) n_others += __shfl_xor(n_others, d, 64);
+    double before = forced_sum, prev_before = 0.0;
+    for (int it = 0; it < kMaxExtract; ++it) {
+      const double mass = one_forced ? (it == 0 ? 0.0 : prev_before) : before;
+      if (!(mass < required) || n_others == 0) {
+        finished = true;
+        dropped = n_others > 0;
+        break;
+      }
+      uint32_t best = 0;
+#pragma unroll
+      for (int u = 0; u < kSlots; ++u) best = vals[u] > best ? vals[u] : best;
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) {
+        const uint32_t o = __shfl_xor(best, d, 64);
+        best = o > best ? o : best;
+      }
+      uint32_t col = 0xffffffffu;     // lowest column holding the maximum
+#pragma unroll
+      for (int u = kSlots - 1; u >= 0; --u) col = vals[u] == best ? (uint32_t)(u * 64 + lane) : col;
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) {
+        const uint32_t o = __shfl_xor(col, d, 64);
+        col = o < col ? o : col;
+      }
+#pragma unroll
+      for (int u = 0; u < kSlots; ++u) vals[u] = (uint32_t)(u * 64 + lane) == col ? 0u : vals[u];
+      if (lane == 0) flags[col] = 1;
+      prev_before = before;
+      before += (double)__uint_as_float(best - 1u);
+      --n_others;
+    }
+  }
+
+  if (!finished) {
+  // ---- bitonic sort, descending
   for (int k = 2; k <= np2; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
       for (int t = lane; t < (np2 >> 1); t += 64) {
@@ -119,7 +184,6 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     if (lane >= d) incl += o;
   }
   double before = forced_sum + (incl - local);
-  int dropped = 0;
   for (int u = 0; u < per; ++u) {
     const int rank = lane * per + u;
     const uint64_t key = keys[rank];
@@ -132,6 +196,7 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     }
     before += key_value(key);
   }
+  }   // sort path
   const bool any_dropped = __any(dropped);
   __syncthreads();
   if (lane == 0) {
