@@ -347,71 +347,92 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   }
 }
 
-// One workgroup = 64 consecutive reshaped query rows (lane <-> row) of one
-// head; its 4 wavefronts split the key range.
+// One workgroup = 64 consecutive reshaped query rows of one head.
+// Pass 1 (lane <-> row, wavefronts split the 128-key tiles) combines the tile
+// maxima / sums into each row's softmax statistics.  Pass 2 rescales the partial
+// block sums and adds the RBS rows of each query block: a lane then owns 4
+// consecutive rows (one 16-byte load per key block), 16 lanes cover the 64 rows
+// and the four lane groups of a wavefront take four key blocks at a time.
 template <int RBS>
 __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
   __shared__ float redM[4][64];
   __shared__ float redL[4][64];
+  __shared__ __attribute__((aligned(16))) float rowM[64];     // row maximum (0 when the row sees nothing)
+  __shared__ __attribute__((aligned(16))) float rowInv[64];   // 1 / row sum, 0 for padded rows
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int head = blockIdx.y;
-  const int m = p.row_begin + blockIdx.x * 64 + lane;
-  const bool row_ok = m < p.row_end;
-  const int mc = row_ok ? m : p.row_end - 1;
-  const int mrel = mc - p.row_begin;
-  const int lo = row_lo(p, mc);
-  int hi = row_hi(p, mc);
-  hi = hi < p.n_rk - 1 ? hi : p.n_rk - 1;
+  const int strip0 = p.row_begin + blockIdx.x * 64;
   const float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
   const float* Mst = p.Mt + (int64_t)head * p.nT * p.rows;
   const float* Lst = p.Lt + (int64_t)head * p.nT * p.rows;
 
-  // pass 1: row statistics from the per-tile maxima and sums
-  float M = -INFINITY, L = 0.f;
-  const int T_lo = lo / kSub, T_hi = hi / kSub;
-  for (int T = T_lo + wave; T <= T_hi; T += 4) {
-    const float mt = Mst[(int64_t)T * p.rows + mrel];
-    const float lt = Lst[(int64_t)T * p.rows + mrel];
-    const float Mn = fmaxf(M, mt);
-    const float safe = (Mn == -INFINITY) ? 0.f : Mn;
-    L = L * fast_exp2(M - safe) + lt * fast_exp2(mt - safe);
-    M = Mn;
+  {
+    const int m = strip0 + lane;
+    const bool row_ok = m < p.row_end;
+    const int mc = row_ok ? m : p.row_end - 1;
+    const int mrel = mc - p.row_begin;
+    const int lo = row_lo(p, mc);
+    int hi = row_hi(p, mc);
+    hi = hi < p.n_rk - 1 ? hi : p.n_rk - 1;
+    float M = -INFINITY, L = 0.f;
+    for (int T = lo / kSub + wave; T <= hi / kSub; T += 4) {
+      const float mt = Mst[(int64_t)T * p.rows + mrel];
+      const float lt = Lst[(int64_t)T * p.rows + mrel];
+      const float Mn = fmaxf(M, mt);
+      const float safe = (Mn == -INFINITY) ? 0.f : Mn;
+      L = L * fast_exp2(M - safe) + lt * fast_exp2(mt - safe);
+      M = Mn;
+    }
+    redM[wave][lane] = M;
+    redL[wave][lane] = L;
+    __syncthreads();
+    if (wave == 0) {
+      const float Mr = fmaxf(fmaxf(redM[0][lane], redM[1][lane]), fmaxf(redM[2][lane], redM[3][lane]));
+      const float safe = (Mr == -INFINITY) ? 0.f : Mr;
+      float Lr = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) Lr += redL[w][lane] * fast_exp2(redM[w][lane] - safe);
+      const bool real = row_ok && mc < p.real_rows && Lr > 0.f;
+      rowM[lane] = safe;
+      rowInv[lane] = real ? 1.f / Lr : 0.f;
+    }
+    __syncthreads();
   }
-  redM[wave][lane] = M;
-  redL[wave][lane] = L;
-  __syncthreads();
-  float Mr = fmaxf(fmaxf(redM[0][lane], redM[1][lane]), fmaxf(redM[2][lane], redM[3][lane]));
-  const float safe = (Mr == -INFINITY) ? 0.f : Mr;
-  float Lr = 0.f;
-#pragma unroll
-  for (int w = 0; w < 4; ++w) Lr += redL[w][lane] * fast_exp2(redM[w][lane] - safe);
-  const bool real = row_ok && mc < p.real_rows && Lr > 0.f;
-  const float inv = real ? 1.f / Lr : 0.f;
 
-  // pass 2: rescale each key block's partial sum and add the RBS rows of a query block
-  const int kb_lo = lo / RBS, kb_hi = hi / RBS;
-  float* out = p.sums + ((int64_t)head * p.nqb + mc / RBS) * p.nkb;
-  // four independent key blocks per trip keep several loads in flight per lane
+  const int l16 = lane & 15, kgrp = lane >> 4;
+  const int m4 = strip0 + l16 * 4;                 // first of this lane's 4 rows
+  const bool rows_ok = m4 < p.row_end;             // row ranges are multiples of 8: all 4 or none
+  const int mc4 = rows_ok ? m4 : p.row_begin;
+  const int mrel4 = mc4 - p.row_begin;
+  const f32x4 rM = *reinterpret_cast<const f32x4*>(rowM + l16 * 4);
+  const f32x4 rI = *reinterpret_cast<const f32x4*>(rowInv + l16 * 4);
+  // the RBS rows of a query block share their first / last visible key block
+  const int kb_lo = row_lo(p, mc4) / RBS;
+  int hi4 = row_hi(p, mc4);
+  hi4 = hi4 < p.n_rk - 1 ? hi4 : p.n_rk - 1;
+  const int kb_hi = hi4 / RBS;
+  float* out = p.sums + ((int64_t)head * p.nqb + mc4 / RBS) * p.nkb;
+  constexpr int kLanesPerBlock = RBS / 4;          // lanes whose 4-row sums make up one query block
+  int T_cached = -1;
+  f32x4 wgt = {0.f, 0.f, 0.f, 0.f};
   for (int kb0 = wave * 4; kb0 < p.nkb; kb0 += 16) {
-    float w[4];
+    const int kb = kb0 + kgrp;
+    float acc = 0.f;
+    if (rows_ok && kb < p.nkb && kb >= kb_lo && kb <= kb_hi) {
+      const int T = (kb * RBS) / kSub;
+      if (T != T_cached) {
+        const f32x4 mt = *reinterpret_cast<const f32x4*>(Mst + (int64_t)T * p.rows + mrel4);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int kb = kb0 + u;
-      w[u] = 0.f;
-      if (real && kb >= kb_lo && kb <= kb_hi && kb < p.nkb) {
-        const int T = (kb * RBS) / kSub;
-        w[u] = Pst[(int64_t)kb * p.rows + mrel] * fast_exp2(Mst[(int64_t)T * p.rows + mrel] - safe) * inv;
+        for (int i = 0; i < 4; ++i) wgt[i] = fast_exp2(mt[i] - rM[i]) * rI[i];
+        T_cached = T;
       }
+      const f32x4 pv = *reinterpret_cast<const f32x4*>(Pst + (int64_t)kb * p.rows + mrel4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc += (rI[i] != 0.f) ? pv[i] * wgt[i] : 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-#pragma unroll
-      for (int d = 1; d < RBS; d <<= 1) w[u] += __shfl_xor(w[u], d, 64);
-    if (row_ok && (lane % RBS) == 0) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (kb0 + u < p.nkb) out[kb0 + u] = w[u];
-    }
+    for (int d = 1; d < kLanesPerBlock; d <<= 1) acc += __shfl_xor(acc, d, 64);
+    if (rows_ok && kb < p.nkb && (l16 % kLanesPerBlock) == 0) out[kb] = acc;
   }
 }
 
