@@ -92,6 +92,41 @@ def cpu_baseline(reps=5, warmup=2):
     }, (q, k, v, mask)
 
 
+def decode_leg(q, k, v, reps=50):
+    """One decode step (the token after the prefill) over the workload's KV cache.
+
+    Not part of the headline value: its own object on the line, with the HBM
+    roofline that bounds it (the step reads K and V once: 2 * H_kv * L * 256 bytes).
+    """
+    import torch
+    from xattn.src import hip_backend
+    from xattn.src.decode import single_decode_with_kv_cache
+
+    lib = hip_backend.lib()
+    heads, kv_heads, L = q.shape[1], k.shape[1], k.shape[2]
+    q1 = q[0, :, -1].contiguous()
+    ws = torch.empty(lib.xattn_decode_workspace_bytes(heads, kv_heads, L), dtype=torch.uint8, device=q.device)
+    out = torch.empty(heads, 128, dtype=q.dtype, device=q.device)
+    for _ in range(5):
+        single_decode_with_kv_cache(q1, k[0], v[0], kv_layout="HND", out=out, workspace=ws)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        single_decode_with_kv_cache(q1, k[0], v[0], kv_layout="HND", out=out, workspace=ws)
+    e1.record()
+    torch.cuda.synchronize()
+    us = _ms(e0, e1) * 1e3 / reps
+    nbytes = 2.0 * kv_heads * L * 256
+    tbs = nbytes / (us * 1e-6) / 1e12
+    return {
+        "kernels": "decode_partial_kernel + decode_merge_kernel",
+        "kv_len": L, "us_per_step": round(us, 1), "bytes": nbytes,
+        "roofline": {"bound": "hbm", "achieved": round(tbs * 1e3, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(tbs * 1e3 / PEAK_HBM_GBS, 4)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -100,6 +135,7 @@ def main():
     ap.add_argument("--workload", type=int, default=2, help="index into the synthetic workloads (default: headline)")
     ap.add_argument("--dense-steps", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode-step measurement")
     ap.add_argument("--compare-pipelined", action="store_true",
                     help="also time Xattention_prefill with and without chunk-by-chunk stream pipelining")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -249,6 +285,8 @@ def main():
         )
         torch.cuda.synchronize()
         del src, dst
+    if not args.no_decode:
+        result["decode_step"] = decode_leg(q, k, v)
     if not args.no_cpu_baseline:
         base, (cq, ck, cv, cmask) = cpu_baseline()
         # the same sample on the GPU path (bf16), for scale

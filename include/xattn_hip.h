@@ -146,6 +146,24 @@ int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* ou
                            int causal, float softmax_scale, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Single-token decode attention over a KV cache.  Replaces the call to the
+ * third-party flashinfer.single_decode_with_kv_cache(q, k, v, kv_layout="HND")
+ * in the reference's Llama attention forward, xattn/src/load_llama.py:191-196:
+ *   out[h] = softmax(q[h] . K[h/g]^T * softmax_scale) V[h/g],  g = H / H_kv <= 32.
+ * q and out are [H][128] (head stride in elements), k and v [H_kv][k_len][128]
+ * with head and token strides in elements (token stride 128..2^22, so both the
+ * "HND" and the "NHD" cache layouts are views).  `workspace` holds the per-range
+ * partial results: at least xattn_decode_workspace_bytes() bytes, 16-byte
+ * aligned, contents undefined on entry and on return.
+ */
+size_t xattn_decode_workspace_bytes(int num_heads, int num_kv_heads, int k_len);
+
+int xattn_decode_fwd(const void* q, const void* k, const void* v, void* out, void* workspace,
+                     size_t workspace_bytes, int num_heads, int num_kv_heads, int k_len, int head_dim,
+                     int64_t q_stride_h, int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h,
+                     int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Measurement aid, no counterpart in the reference: copies `bytes` (a multiple
  * of 16) from src to dst with a plain kernel, i.e. reads `bytes` and writes
  * `bytes` of HBM.  Profiling runs use it to scale hardware byte counters.

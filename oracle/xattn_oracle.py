@@ -19,6 +19,10 @@ follows (paths relative to the reference checkout):
                                      restated as dense softmax attention under
                                      the expanded block mask (and token-causal).
 * :func:`Xattention_prefill`       - xattn/src/Xattention.py:302-402
+* :func:`single_decode_with_kv_cache` - the un-vendored ``flashinfer==0.1.6``
+                                     call at xattn/src/load_llama.py:191-196,
+                                     restated as one softmax attention row per
+                                     query head over the whole cache.
 
 Pinning status (what independent evidence each function is checked against,
 see tests/test_oracle_*.py):
@@ -38,6 +42,10 @@ see tests/test_oracle_*.py):
   results for it).  It is pinned to the mathematics only: all-True mask ==
   torch scaled_dot_product_attention, and a per-row python loop on tiny
   inputs.
+* single_decode_with_kv_cache: PARITY UNPINNED against flashinfer itself
+  (third-party CUDA, absent from the reference tree and from this image).
+  Pinned to the mathematics: equals torch scaled_dot_product_attention with
+  repeated KV heads, and the last row of causal prefill attention.
 * xattn_estimate / Xattention_prefill glue: invariants (block-tril, forced
   sink/diagonal, keep_sink row, keep_recent diagonal) and tiny hand cases.
 """
@@ -395,3 +403,29 @@ def Xattention_prefill(
         query_states, key_states, value_states, mask, causal=causal, block_size=block_size
     )
     return (out, mask) if return_mask else out
+
+
+# --------------------------------------------------------------------------- #
+# decode step
+# --------------------------------------------------------------------------- #
+def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None):
+    """One query token per head against the whole KV cache, fp32 throughout.
+
+    The reference calls flashinfer.single_decode_with_kv_cache(q, k, v,
+    kv_layout="HND") (xattn/src/load_llama.py:191-196) with q ``[H, d]`` and
+    k, v ``[H_kv, L, d]``; query head h reads KV head ``h // (H / H_kv)``, the
+    scale defaults to ``1/sqrt(d)``, no positional transform is applied.
+    Returns ``[H, d]`` in q's dtype.
+    """
+    if kv_layout == "NHD":
+        k, v = k.transpose(0, 1), v.transpose(0, 1)
+    heads, dim = q.shape
+    group = heads // k.shape[0]
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(dim)
+    out = torch.empty((heads, dim), dtype=torch.float32)
+    for h in range(heads):
+        kh = k[h // group].float()
+        logits = (kh @ q[h].float()) * sm_scale
+        out[h] = torch.softmax(logits, dim=0) @ v[h // group].float()
+    return out.to(q.dtype)

@@ -25,6 +25,11 @@ _SIGNATURES = {
         [c_vp] * 5 + [c_i64] + [c_i32] * 13 + [c_vp],
     ),
     "xattn_calibration_copy": (c_i32, [c_vp, c_vp, c_sz, c_vp]),
+    "xattn_decode_workspace_bytes": (c_sz, [c_i32] * 3),
+    "xattn_decode_fwd": (
+        c_i32,
+        [c_vp] * 5 + [c_sz] + [c_i32] * 4 + [c_i64] * 6 + [c_f32, c_vp],
+    ),
     "xattn_block_sparse_fwd": (
         c_i32,
         [c_vp] * 6 + [c_i64] + [c_i32] * 6 + [c_i64] * 8 + [c_i32, c_i32, c_i32, c_f32, c_vp],
