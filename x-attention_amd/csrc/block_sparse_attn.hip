@@ -28,6 +28,7 @@ namespace xattn {
 
 constexpr int kBlk = 128;          // block_size of the operator
 constexpr int kTileBytes = kBlk * 256;   // one K or V tile in LDS
+constexpr int kUnit = 64;                // workgroups resident on one XCD (32 CUs x 2)
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4;
@@ -44,6 +45,7 @@ struct AttnParams {
   int idx_rows;             // q-block rows per head in col_idx / col_cnt (>= nqb)
   int H, Hkv, Lq, Lk, nqb, nkb;
   int qb_begin, qb_end;     // q-blocks handled by this launch
+  int unit_rows;            // q-blocks per dispatch unit
   int causal, kv_off;       // kv_off = Lk - Lq
   float scale_log2;         // softmax_scale * log2(e)
 };
@@ -89,21 +91,27 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
 
-  // Workgroup ids are dealt round-robin to the 8 XCDs.  Eight consecutive ids
-  // take eight consecutive q-blocks of ONE head, so every head's rows - whose
-  // list lengths vary smoothly with the row but by orders of magnitude between
-  // heads - are spread evenly over the XCDs; the next eight ids take the next
-  // head, so the query heads of a KV group with the same q-block run side by
-  // side on one XCD and share its L2 for K/V.  Rows go out last (longest, when
-  // causal) first.
+  // Workgroup ids are dealt round-robin to the 8 XCDs, and an XCD (32 CUs, two
+  // workgroups each, one L2) starts its workgroups in id order.  The 64 ids that
+  // land on one XCD one after the other form a unit: the query heads of ONE KV
+  // head times a run of adjacent q-blocks, so everything resident on the XCD
+  // streams the same K/V through its L2 at about the same place.  Units are
+  // dealt to XCDs in turn; the KV head of a unit rotates with the q-block run,
+  // so every XCD sees every head equally often (heads differ by orders of
+  // magnitude in list length).  Runs go out last (longest, when causal) first.
   int head, qb;
   {
+    const int group = p.H / p.Hkv;
+    const int G = p.unit_rows;                 // q-blocks per unit, group * G = kUnit
     const int id = blockIdx.x;
     const int x = id & 7, s = id >> 3;
-    head = s % p.H;
-    const int from_end = (s / p.H) * 8 + x;
-    if (from_end >= p.qb_end - p.qb_begin) return;
+    const int unit = (s / kUnit) * 8 + x, w = s % kUnit;
+    const int run = unit / p.Hkv;
+    const int kvh_u = (unit % p.Hkv + run) % p.Hkv;
+    const int from_end = run * G + w / group;
+    if (w >= group * G || from_end >= p.qb_end - p.qb_begin) return;
     qb = p.qb_end - 1 - from_end;
+    head = kvh_u * group + w % group;
   }
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
@@ -376,7 +384,11 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   if (q_block_begin < 0 || q_block_begin >= q_block_end || q_block_end > p.nqb) return XATTN_ERR_SHAPE;
   p.qb_begin = q_block_begin;
   p.qb_end = q_block_end;
-  const int64_t grid = (int64_t)p.H * ((q_block_end - q_block_begin + 7) / 8) * 8;
+  const int group = p.H / p.Hkv;
+  p.unit_rows = group >= kUnit ? 1 : kUnit / group;
+  const int64_t runs = (q_block_end - q_block_begin + p.unit_rows - 1) / p.unit_rows;
+  const int64_t units = (runs * p.Hkv + 7) / 8 * 8;
+  const int64_t grid = units * kUnit;
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
   if (col_idx)
     hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(256), 0,

@@ -8,7 +8,7 @@
 //  kernel 1 (estimate_gemm_kernel): a bf16 MFMA GEMM over the reshaped
 //    operands, gathered on the fly - reshaped key n at depth slab i is token
 //    n*S+i, reshaped query m is token m*S+S-1-i - with a 256x256 tile per
-//    workgroup and 128x128 per wavefront.  Scores are produced transposed
+//    workgroup of eight wavefronts, 128 keys x 64 query rows each.  Scores are produced transposed
 //    (keys along accumulator rows) so one lane owns one query row.  In the
 //    epilogue each wavefront scales, masks, takes the row maximum over ITS 128
 //    keys, exponentiates against that local maximum and adds up groups of
@@ -24,7 +24,9 @@
 namespace xattn {
 
 constexpr int kTile = 256;       // workgroup tile edge (reshaped rows / keys)
-constexpr int kSub = 128;        // wavefront tile edge
+constexpr int kSub = 128;        // keys per wavefront tile (and per softmax tile)
+constexpr int kRowsW = 64;       // reshaped query rows per wavefront tile
+constexpr int kWaves = 8;        // wavefronts per workgroup: 2 key halves x 4 query quarters
 constexpr int kDepth = 64;       // bf16 per k-step (one 128-byte line per row)
 constexpr int kStageBytes = 2 * kTile * kDepth * 2;  // K' + Q' slabs of one stage
 
@@ -75,26 +77,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // Per-lane byte offsets (relative to the tile's first token) of the 8 rows a
 // lane copies per slab, for token 0 of each reshaped row's group and feature 0;
 // the k-step adds a uniform term.  The host checks that a tile spans < 2^31 bytes.
-__device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int S, int lane, int wave, int (&voff)[8]) {
+__device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int S, int lane, int wave, int (&voff)[4]) {
   const int c = lane & 7, rl = lane >> 3;
 #pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int r = it * 32 + wave * 8 + rl;
+  for (int it = 0; it < 4; ++it) {
+    const int r = it * 64 + wave * 8 + rl;
     voff[it] = (int)((int64_t)r * S * sn_bytes) + ((c ^ ((r >> 1) & 7)) << 4);
   }
 }
 
-__device__ __forceinline__ void copy_slab(__amdgpu_buffer_rsrc_t rsrc, const int (&voff)[8], int step_off,
-                                          char* slab, int wave) {
-#pragma unroll
-  for (int it = 0; it < 8; ++it)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 32 + wave * 8) * 128), 16,
-                                             (int)((unsigned)voff[it] + (unsigned)step_off), 0, 0, 0);
-}
-
 __device__ __forceinline__ void copy_one(__amdgpu_buffer_rsrc_t rsrc, int voff, int step_off, char* slab, int wave,
                                          int it) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 32 + wave * 8) * 128), 16,
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 64 + wave * 8) * 128), 16,
                                            (int)((unsigned)voff + (unsigned)step_off), 0, 0, 0);
 }
 
@@ -105,12 +99,13 @@ __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk
 
 // kDump: also write the raw scores (test / seam builds only; kept out of the production instantiation)
 template <int RBS, bool kDump>
-__global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
+__global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, hh = lane >> 5;
-  const int wm = wave & 1, wn = wave >> 1;
+  const int wm = wave & 3, wn = wave >> 2;   // query quarter, key half
   // Tile assignment.  Only tiles holding a visible (row, key) pair are
   // enumerated: per KV group, by query tile row, then key tile, then query head
   // of the group.  Workgroup ids are dealt round-robin to the 8 XCDs, so runs of
@@ -168,51 +163,50 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(kbase + (k_rows > 0 ? k_tok0 * p.k_sn : 0)), 0, (int)(k_rows * k_snb), 0x00020000);
 
-  f32x16 acc[4][4];   // [key tile nt][query tile mt]
+  f32x16 acc[4][2];   // [key tile nt][query tile mt]
 #pragma unroll
   for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+    for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
   // k-step t covers token i = t / 2 of every reshaped row's group, features
   // 64*(t % 2) .. +63, and is read from LDS stage t % 2.
   //
-  // Software pipeline.  A step is four sub-steps of 16 MFMAs; the 8 fragment
-  // reads of the next sub-step and 4 of the 16 copies of a later step are
-  // issued between them, in chunks the scheduler may not mix (one copy, two
-  // reads, four MFMAs: with one wavefront per SIMD issue is in order, so a burst
-  // of copies or reads would hold back the MFMAs queued behind it).  The
-  // workgroup barrier sits before the LAST sub-step's MFMAs: at that point every
-  // fragment of the current stage has been read, so the sub-step can prefetch
-  // the next stage's first fragments and start refilling the current stage
-  // while its MFMAs run - the MFMA stream never drains at a step boundary.
+  // Software pipeline.  A step is four sub-steps of 8 MFMAs per wavefront; the 6
+  // fragment reads of the next sub-step and 2 of the 8 copies of a later step
+  // are issued between them, in chunks the scheduler may not mix (one copy, two
+  // reads, two MFMAs), so that neither copies nor reads bunch up in front of the
+  // MFMAs.  Two wavefronts share a SIMD: while one waits at the barrier or on a
+  // fragment the other keeps the matrix pipe fed.  The workgroup barrier sits
+  // before the LAST sub-step's MFMAs: at that point every fragment of the
+  // current stage has been read, so the sub-step can prefetch the next stage's
+  // first fragments and start refilling the current stage while its MFMAs run.
   const int steps = p.S * 2;
-  int voffK[8], voffQ[8];
+  int voffK[4], voffQ[4];
   slab_offsets(k_snb, p.S, lane, wave, voffK);
   slab_offsets(q_snb, p.S, lane, wave, voffQ);
   auto step_off_k = [&](int t) { return (t >> 1) * (int)k_snb + (t & 1) * kDepth * 2; };
   auto step_off_q = [&](int t) { return (p.S - 1 - (t >> 1)) * (int)q_snb + (t & 1) * kDepth * 2; };
-  // copy j (0..15) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
+  // copy j (0..7) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
   auto copy_j = [&](int j, int t, char* stage) {
     const int tc = t < steps ? t : steps - 1;       // past the end: a harmless repeat
     if (j & 1) copy_one(qres, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
     else copy_one(kres, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
   };
 #pragma unroll
-  for (int j = 0; j < 16; ++j) copy_j(j, 0, lds);
+  for (int j = 0; j < 8; ++j) copy_j(j, 0, lds);
   wait_vm0();
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < 4; ++j) copy_j(j, 1, lds + kStageBytes);
+  for (int j = 0; j < 2; ++j) copy_j(j, 1, lds + kStageBytes);
 
-  bf16x8 fa[2][4], fb[2][4];
+  bf16x8 fa[2][4], fb[2][2];
 #pragma unroll
-  for (int x = 0; x < 4; ++x) {
-    fa[0][x] = read_frag(lds, wn * kSub + x * 32 + r, hh);
-    fb[0][x] = read_frag(lds + kTile * 128, wm * kSub + x * 32 + r, hh);
-  }
+  for (int x = 0; x < 4; ++x) fa[0][x] = read_frag(lds, wn * kSub + x * 32 + r, hh);
+#pragma unroll
+  for (int x = 0; x < 2; ++x) fb[0][x] = read_frag(lds + kTile * 128, wm * kRowsW + x * 32 + r, hh);
 
   for (int t = 0; t < steps; ++t) {
     char* cur = lds + (t & 1) * kStageBytes;
@@ -232,24 +226,24 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         __builtin_amdgcn_sched_barrier(0);
-        if (ss < 3) copy_j(4 + ss * 4 + c, t + 1, nxt);    // copies 4..15 of step t+1
-        else copy_j(c, t + 2, cur);                        // copies 0..3 of step t+2 refill this stage
         if (c < 2) {
+          if (ss < 3) copy_j(2 + ss * 2 + c, t + 1, nxt);  // copies 2..7 of step t+1
+          else copy_j(c, t + 2, cur);                      // copies 0..1 of step t+2 refill this stage
           fa[(ss + 1) & 1][2 * c] = read_frag(fragK, wn * kSub + (2 * c) * 32 + r, nss * 2 + hh);
           fa[(ss + 1) & 1][2 * c + 1] = read_frag(fragK, wn * kSub + (2 * c + 1) * 32 + r, nss * 2 + hh);
-        } else {
-          fb[(ss + 1) & 1][2 * c - 4] = read_frag(fragQ, wm * kSub + (2 * c - 4) * 32 + r, nss * 2 + hh);
-          fb[(ss + 1) & 1][2 * c - 3] = read_frag(fragQ, wm * kSub + (2 * c - 3) * 32 + r, nss * 2 + hh);
+        } else if (c == 2) {
+          fb[(ss + 1) & 1][0] = read_frag(fragQ, wm * kRowsW + r, nss * 2 + hh);
+          fb[(ss + 1) & 1][1] = read_frag(fragQ, wm * kRowsW + 32 + r, nss * 2 + hh);
         }
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[c][mt] = mfma32(fa[ss & 1][c], fb[ss & 1][mt], acc[c][mt]);
+        for (int mt = 0; mt < 2; ++mt) acc[c][mt] = mfma32(fa[ss & 1][c], fb[ss & 1][mt], acc[c][mt]);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
   wait_vm0();   // the repeats issued by the last steps
 
-  // ---- epilogue: this wavefront's 128 keys x 128 query rows
+  // ---- epilogue: this wavefront's 128 keys x 64 query rows
   const int nbase = n0 + wn * kSub;       // first key of the wavefront tile
   const int T = nbase / kSub;
   if (nbase >= p.n_rk) return;
@@ -258,12 +252,12 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
   float* Lst = p.Lt + ((int64_t)head * p.nT + T) * p.rows;
   // every key of this wavefront tile visible to every one of its query rows?
   // (true away from the diagonal and the sequence end: no per-element masking)
-  const int mw0 = m0 + wm * kSub;
+  const int mw0 = m0 + wm * kRowsW;
   const bool all_visible = nbase + kSub <= p.n_rk && nbase + kSub - 1 <= row_hi(p, mw0) &&
-                           nbase >= row_lo(p, mw0 + kSub - 1);
+                           nbase >= row_lo(p, mw0 + kRowsW - 1);
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int m = m0 + wm * kSub + mt * 32 + r;
+  for (int mt = 0; mt < 2; ++mt) {
+    const int m = m0 + wm * kRowsW + mt * 32 + r;
     const bool row_ok = m < p.row_end;
     const int lo = row_lo(p, m), hi = row_hi(p, m);
     if (kDump && row_ok) {
@@ -341,8 +335,7 @@ __global__ __launch_bounds__(256, 1) void estimate_gemm_kernel(EstParams p) {
       Mst[mrel] = mx;
       Lst[mrel] = tot;
     }
-    // keep the four query-tile passes apart: interleaving them only lengthens
-    // live ranges on top of the 256 accumulator registers
+    // keep the query-tile passes apart: interleaving them only lengthens live ranges
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -447,7 +440,7 @@ hipError_t launch_gemm(const EstParams& p, dim3 grid, size_t lds, hipStream_t s)
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, grid, dim3(256), lds, s, p);
+  hipLaunchKernelGGL(kernel, grid, dim3(kWaves * 64), lds, s, p);
   return hipSuccess;
 }
 
