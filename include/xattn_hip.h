@@ -164,6 +164,37 @@ int xattn_decode_fwd(const void* q, const void* k, const void* v, void* out, voi
                      int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Threshold profiler, xattn/threshold/profile_threshold/profile_threshold.py.
+ *
+ * xattn_block_mass replaces chunk_prefill_to_attn_sum (:15-57): the true
+ * softmax(q k^T * softmax_scale) probabilities (token-causal when `causal`,
+ * bottom-right aligned when k_len > q_len; the reference always masks
+ * causally and asserts equal block counts) summed over each 128 x 128 block,
+ *   mass[h][i][j] = sum over rows of q-block i, keys of k-block j,
+ * fp32 [H][ceil(q_len/128)][ceil(k_len/128)], every entry written (zeros for
+ * blocks no row of the q-block sees).  Rows past q_len carry no mass, so a
+ * full q-block row of `mass` sums to 128.  Nothing is materialised.
+ *
+ * xattn_threshold_rows does the per-row part of xattn_prefill_profile
+ * (:84-93): for (head, q-block row) it takes blocks by decreasing mass until
+ * `coverage` (0.9 in the reference) of the row's mass is reached, including the
+ * block that crosses, finds the smallest estimate_sums value among them and
+ * writes rows_out[h][i] = { sum of the row's estimate_sums at or above that
+ * value, sum of the row's estimate_sums }.  The profiled threshold of head h is
+ * sum_i rows_out[h][i][0] / (sum_i rows_out[h][i][1] + 1e-8) (:93); the caller
+ * adds the rows up.  estimate_sums is read as [h * est_head_pitch +
+ * i * est_row_pitch + j] (elements), so the padded output of
+ * xattn_estimate_block_sums can be passed as it is.  nk_blocks <= 16384.
+ */
+int xattn_block_mass(const void* q, const void* k, float* mass, int num_heads, int num_kv_heads,
+                     int q_len, int k_len, int head_dim, int64_t q_stride_h, int64_t q_stride_n,
+                     int64_t k_stride_h, int64_t k_stride_n, int causal, float softmax_scale, void* stream);
+
+int xattn_threshold_rows(const float* block_mass, const float* estimate_sums, float* rows_out,
+                         int num_heads, int nq_blocks, int nk_blocks, int64_t est_head_pitch,
+                         int64_t est_row_pitch, float coverage, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Measurement aid, no counterpart in the reference: copies `bytes` (a multiple
  * of 16) from src to dst with a plain kernel, i.e. reads `bytes` and writes
  * `bytes` of HBM.  Profiling runs use it to scale hardware byte counters.

@@ -19,6 +19,9 @@ follows (paths relative to the reference checkout):
                                      restated as dense softmax attention under
                                      the expanded block mask (and token-causal).
 * :func:`Xattention_prefill`       - xattn/src/Xattention.py:302-402
+* :func:`chunk_prefill_to_attn_sum`,
+  :func:`profile_threshold_head`   - xattn/threshold/profile_threshold/
+                                     profile_threshold.py:15-57 and :84-93
 * :func:`single_decode_with_kv_cache` - the un-vendored ``flashinfer==0.1.6``
                                      call at xattn/src/load_llama.py:191-196,
                                      restated as one softmax attention row per
@@ -46,6 +49,12 @@ see tests/test_oracle_*.py):
   (third-party CUDA, absent from the reference tree and from this image).
   Pinned to the mathematics: equals torch scaled_dot_product_attention with
   repeated KV heads, and the last row of causal prefill attention.
+* chunk_prefill_to_attn_sum: a full softmax matrix on tiny inputs summed per
+  block by a python loop; every real q-block row sums to its number of rows.
+  profile_threshold_head: a hand-worked example and a python re-derivation
+  from the definition (fewest blocks reaching the coverage, minimum estimate
+  among them, share of the estimate at or above it).  The reference module
+  itself needs flash_attn and a GPU at import and cannot be run here.
 * xattn_estimate / Xattention_prefill glue: invariants (block-tril, forced
   sink/diagonal, keep_sink row, keep_recent diagonal) and tiny hand cases.
 """
@@ -429,3 +438,47 @@ def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None):
         logits = (kh @ q[h].float()) * sm_scale
         out[h] = torch.softmax(logits, dim=0) @ v[h // group].float()
     return out.to(q.dtype)
+
+
+# --------------------------------------------------------------------------- #
+# threshold profiler
+# --------------------------------------------------------------------------- #
+def chunk_prefill_to_attn_sum(query_states, key_states, block_size=128):
+    """True causal attention mass per block, ``[B, H, Nq, Nk]`` fp32.
+
+    Follows xattn/threshold/profile_threshold/profile_threshold.py:15-57 with
+    fp32 arithmetic: q-block by q-block, ``softmax(q k^T / sqrt(d))`` over the
+    keys at or before each query (keys and query rows past the end excluded),
+    summed over the block's rows and over each key block.  GQA by head sharing.
+    """
+    bsz, heads, q_len, d = query_states.shape
+    kv_heads, k_len = key_states.shape[1], key_states.shape[2]
+    assert q_len == k_len
+    group = heads // kv_heads
+    nb = (q_len + block_size - 1) // block_size
+    k = key_states.float().repeat_interleave(group, 1)
+    out = torch.zeros((bsz, heads, nb, nb), dtype=torch.float32)
+    pos_k = torch.arange(nb * block_size)
+    for i in range(nb):
+        rows = torch.arange(i * block_size, min((i + 1) * block_size, q_len))
+        w = torch.matmul(query_states[:, :, rows].float(), k.transpose(2, 3)) / math.sqrt(d)
+        w = F.pad(w, (0, nb * block_size - k_len), value=NEG_INF)
+        dead = (pos_k[None, :] > rows[:, None]) | (pos_k[None, :] >= k_len)
+        w = w.masked_fill(dead, NEG_INF)
+        p = F.softmax(w, dim=-1, dtype=torch.float32)
+        out[:, :, i] = p.view(bsz, heads, len(rows), nb, block_size).sum(-1).sum(-2)
+    return out
+
+
+def profile_threshold_head(attn_sum, xattn_sum, coverage=0.9):
+    """``[B, H]`` thresholds, profile_threshold.py:84-93 (``xattn_sum`` already
+    cropped to ``attn_sum``'s shape and multiplied by the stride)."""
+    vals, idx = torch.sort(attn_sum, dim=-1, descending=True, stable=True)
+    cumsum = vals.cumsum(-1)
+    need_len = (cumsum < coverage * cumsum[..., -1:]).sum(-1) + 1
+    rank = torch.arange(vals.size(-1))
+    selected = rank.view(1, 1, 1, -1) < need_len.unsqueeze(-1)
+    x_sorted = xattn_sum.gather(-1, idx)
+    miniblock = x_sorted.masked_fill(~selected, float("inf")).min(-1).values
+    at_or_above = xattn_sum >= miniblock.unsqueeze(-1)
+    return (xattn_sum * at_or_above).sum(-1).sum(-1) / (xattn_sum.sum(-1).sum(-1) + 1e-8)

@@ -21,17 +21,10 @@
 // K tile overlaps softmax and P.V, the copy of the next V tile overlaps Q.K^T.
 // Two workgroups fit per CU (64 KiB LDS each) so one's softmax overlaps the
 // other's MFMA.
-#include "xattn_common.h"
+#include "attn_tiles.h"
 #include "xattn_hip.h"
 
 namespace xattn {
-
-constexpr int kBlk = 128;          // block_size of the operator
-constexpr int kTileBytes = kBlk * 256;   // one K or V tile in LDS
-constexpr int kUnit = 64;                // workgroups resident on one XCD (32 CUs x 2)
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef __attribute__((__vector_size__(4 * sizeof(short)))) short i16x4;
 
 struct AttnParams {
   const __bf16* q;
@@ -52,36 +45,6 @@ struct AttnParams {
 
 __device__ __forceinline__ int clamp_block(int kb, int nkb) { return kb < 0 ? 0 : (kb < nkb ? kb : nkb - 1); }
 
-// LDS tile layout: row n at byte n*256, its 16-byte chunk c stored at chunk
-// c ^ swz(n).  swz takes all 16 values over 16 consecutive rows (row-per-lane
-// b128 reads of one logical chunk are conflict-free) and moves rows n..n+3 into
-// different 64-byte groups (the 4-row x 32-byte gathers of the transposing read
-// are conflict-free too).
-__device__ __forceinline__ int swz(int n) { return ((n & 3) << 2) | ((n >> 2) & 3); }
-
-// Copies key block kb of one head (row stride sn elements) into an LDS tile.
-// Wavefront w issues 8 instructions of 1 KiB (4 rows) each; voff[i] is the
-// lane's byte offset inside the block for instruction i.
-__device__ __forceinline__ void copy_tile(const __bf16* base, int64_t sn, int len, int kb, const int (&voff)[8],
-                                          char* tile, int wave) {
-  const int rows_left = len - kb * kBlk;
-  const int rows = rows_left < kBlk ? rows_left : kBlk;
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(base + (int64_t)kb * kBlk * sn), 0, (int)((int64_t)rows * sn * 2), 0x00020000);
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(tile + (wave * 8 + i) * 1024), 16, voff[i], 0, 0, 0);
-}
-
-__device__ __forceinline__ void tile_offsets(int64_t sn, int lane, int wave, int (&voff)[8]) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = 4 * (wave * 8 + i) + (lane >> 4);
-    const int c = (lane & 15) ^ swz(row);
-    voff[i] = (int)(row * sn * 2) + (c << 4);
-  }
-}
-
 // kHasList = false is the dense baseline (its own symbol, so profiles tell the two apart)
 template <bool kHasList>
 __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) {
@@ -91,28 +54,8 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
 
-  // Workgroup ids are dealt round-robin to the 8 XCDs, and an XCD (32 CUs, two
-  // workgroups each, one L2) starts its workgroups in id order.  The 64 ids that
-  // land on one XCD one after the other form a unit: the query heads of ONE KV
-  // head times a run of adjacent q-blocks, so everything resident on the XCD
-  // streams the same K/V through its L2 at about the same place.  Units are
-  // dealt to XCDs in turn; the KV head of a unit rotates with the q-block run,
-  // so every XCD sees every head equally often (heads differ by orders of
-  // magnitude in list length).  Runs go out last (longest, when causal) first.
   int head, qb;
-  {
-    const int group = p.H / p.Hkv;
-    const int G = p.unit_rows;                 // q-blocks per unit, group * G = kUnit
-    const int id = blockIdx.x;
-    const int x = id & 7, s = id >> 3;
-    const int unit = (s / kUnit) * 8 + x, w = s % kUnit;
-    const int run = unit / p.Hkv;
-    const int kvh_u = (unit % p.Hkv + run) % p.Hkv;
-    const int from_end = run * G + w / group;
-    if (w >= group * G || from_end >= p.qb_end - p.qb_begin) return;
-    qb = p.qb_end - 1 - from_end;
-    head = kvh_u * group + w % group;
-  }
+  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, p.unit_rows, p.qb_begin, p.qb_end, &head, &qb)) return;
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
@@ -384,11 +327,8 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   if (q_block_begin < 0 || q_block_begin >= q_block_end || q_block_end > p.nqb) return XATTN_ERR_SHAPE;
   p.qb_begin = q_block_begin;
   p.qb_end = q_block_end;
-  const int group = p.H / p.Hkv;
-  p.unit_rows = group >= kUnit ? 1 : kUnit / group;
-  const int64_t runs = (q_block_end - q_block_begin + p.unit_rows - 1) / p.unit_rows;
-  const int64_t units = (runs * p.Hkv + 7) / 8 * 8;
-  const int64_t grid = units * kUnit;
+  p.unit_rows = unit_rows_for(p.H, p.Hkv);
+  const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
   if (col_idx)
     hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(256), 0,
