@@ -72,6 +72,17 @@ const char* xattn_error_string(int code);
  * `scores_out`, when non-null, receives the un-scaled scores of those chunks as
  * fp32 [num_heads][n_rq][n_rk] (entries of tiles with no visible pair are left
  * untouched) - the flat_group_gemm_fuse_reshape seam, for tests.
+ * `slab_pairs` (HOST pointer, 2 * num_slab_pairs ints, at most 64 pairs; NULL /
+ * 0 for the default) generalises the reshape to the reference's other
+ * select_mode settings (torch branch only, Xattention.py:72-135): the score is
+ *   sum over pairs (a, b) of Q[m*stride + a] . K[n*stride + b],
+ * the default being the pairs (stride-1-i, i).  "slash" is (i, i); "random"
+ * (perm[i], i); "double" adds (stride-1-i, (i+1) % stride); "triple" weights
+ * (stride-1-i, i) twice and adds (stride-1-i, (i+1) % stride) and
+ * (stride-1-i, (i-1) % stride) (the reference adds the rolled key slabs in the
+ * input precision before the product, this sum is taken in fp32).
+ * softmax == 0 writes block sums of exp(scaled score) over the visible keys
+ * instead of softmax probabilities (Xattention.py:231-234).
  * `workspace` must hold xattn_estimate_workspace_bytes(...) bytes, where
  * chunks_per_call is the largest chunk_end - chunk_begin used (<= 0: all chunks);
  * the function returns 0 for arguments the estimator rejects.
@@ -84,7 +95,8 @@ int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, v
                               int num_kv_heads, int q_len, int k_len, int head_dim, int64_t q_stride_h,
                               int64_t q_stride_n, int64_t k_stride_h, int64_t k_stride_n, int stride,
                               int block_size, int chunk_size, int chunk_begin, int chunk_end, int causal,
-                              int own_chunk_only, float scale, void* stream);
+                              int own_chunk_only, float scale, const int32_t* slab_pairs,
+                              int num_slab_pairs, int softmax, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Threshold block selection.  Replaces find_blocks_chunked,

@@ -84,6 +84,29 @@ def reshape_inverse(query_states, key_states, stride):
     return rq, rk
 
 
+def reshape_operands(query_states, key_states, stride, select_mode="inverse", perm=None):
+    """The reshaped (query, key) pair of every ``select_mode`` of the torch
+    branch, xattn/src/Xattention.py:72-135 (``kdb=1``).  ``perm`` stands for the
+    ``torch.randperm(stride)`` the reference draws for "random"."""
+    S, d = stride, query_states.shape[-1]
+    rk = torch.cat([key_states[:, :, i::S, :] for i in range(S)], dim=-1)
+    if select_mode in ("inverse", ""):
+        return reshape_inverse(query_states, key_states, stride)
+    if select_mode == "random":
+        rq = torch.cat([query_states[:, :, int(perm[i]) :: S, :] for i in range(S)], dim=-1)
+        return rq, rk
+    if select_mode == "slash":
+        rq = torch.cat([query_states[:, :, i::S, :] for i in range(S)], dim=-1)
+        return rq, rk
+    rq = torch.cat([query_states[:, :, (S - 1 - i) :: S, :] for i in range(S)], dim=-1)
+    if select_mode in ("double", "triple"):
+        rk = rk + torch.cat([rk[..., d:], rk[..., :d]], dim=-1)
+        if select_mode == "triple":
+            rk = rk + torch.cat([rk[..., -d:], rk[..., :-d]], dim=-1)
+        return rq, rk
+    raise ValueError(select_mode)
+
+
 def antidiagonal_scores(query_states, key_states, stride):
     """score[m, n] = sum_i Q[m*S + S-1-i] . K[n*S + i]  (un-scaled).
 
@@ -188,6 +211,7 @@ def estimate_chunk_block_sums(
     causal,
     pad0_quirk,
     out_dtype,
+    softmax=True,
 ):
     """Block sums of softmax(antidiagonal scores) for one query chunk.
 
@@ -219,7 +243,10 @@ def estimate_chunk_block_sums(
             cm[:, :, (-q_reshaped_num_to_pad):, :] = NEG_INF
         cm[..., c1:] = NEG_INF
         w = w + cm
-    w = F.softmax(w, dim=-1, dtype=torch.float32).to(out_dtype)
+    if softmax:
+        w = F.softmax(w, dim=-1, dtype=torch.float32).to(out_dtype)
+    else:
+        w = torch.exp(w).to(out_dtype)   # Xattention.py:231-234
     if last_padded:
         w[:, :, (-q_reshaped_num_to_pad):, :] = 0
     sums = w.view(bsz, heads, rcs // rbs, rbs, -1, rbs).sum(dim=-1).sum(dim=-2)
@@ -242,17 +269,18 @@ def xattn_estimate(
     keep_sink=False,
     keep_recent=False,
     pad0_quirk=True,
+    perm=None,
 ):
     """(attn_sums, simple_masks), both ``[B, H, Nq_blocks_padded, Nk_blocks_padded]``.
 
-    Restates xattn/src/Xattention.py:13-299 for ``select_mode="inverse"``,
-    ``kdb=1``, ``softmax=True`` on whatever device the inputs live on.
+    Restates xattn/src/Xattention.py:13-299 for ``kdb=1`` on whatever device
+    the inputs live on (``perm``: the permutation "random" would draw).
     ``use_triton`` is accepted for signature parity and ignored; the only
     semantic difference between the two upstream branches that survives in
     exact arithmetic is ``pad0_quirk`` (see :func:`estimate_chunk_block_sums`).
     """
-    if select_mode not in ("inverse", "") or kdb != 1 or not softmax:
-        raise NotImplementedError("only select_mode='inverse', kdb=1, softmax=True")
+    if kdb != 1:
+        raise NotImplementedError("only kdb=1")
     bsz, kv_heads, k_len, head_dim = key_states.shape
     _, heads, q_len, _ = query_states.shape
     assert heads == kv_heads
@@ -266,7 +294,7 @@ def xattn_estimate(
     assert k_chunk_num >= q_chunk_num
     pk = F.pad(key_states, (0, 0, 0, k_pad), value=0) if k_pad else key_states
     pq = F.pad(query_states, (0, 0, 0, q_pad), value=0) if q_pad else query_states
-    rq, rk = reshape_inverse(pq, pk, stride)
+    rq, rk = reshape_operands(pq, pk, stride, select_mode, perm)
     blocks_per_chunk = chunk_size // block_size
 
     sums, masks = [], []
@@ -287,6 +315,7 @@ def xattn_estimate(
             causal=causal,
             pad0_quirk=pad0_quirk,
             out_dtype=pq.dtype,
+            softmax=softmax,
         )
         m = find_blocks_chunked(
             s,

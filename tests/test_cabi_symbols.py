@@ -56,12 +56,12 @@ def test_operator_refuses_cpu_tensors_and_wrong_dtypes():
     q = torch.zeros(1, 2, 256, 128, dtype=torch.bfloat16)
     with pytest.raises(hb.XattnHipError):
         Xattention_prefill(q, q, q, 8)
-    with pytest.raises(NotImplementedError):
-        xattn_estimate(q, q, 128, 8, select_mode="slash")
+    with pytest.raises(ValueError):
+        xattn_estimate(q, q, 128, 8, select_mode="diagonal")     # not one of the reference's modes
     with pytest.raises(ValueError):
         xattn_estimate(q, q, 128, 8, kdb=2)
-    with pytest.raises(NotImplementedError):
-        xattn_estimate(q, q, 128, 8, softmax=False)
+    with pytest.raises(hb.XattnHipError):
+        xattn_estimate(q, q, 128, 8, select_mode="slash", softmax=False)   # valid request, CPU tensors
     table = {1024: 2048, 4096: 4096, 16384: 16384, 32768: 8192, 65536: 4096, 131072: 2048, 119056: 2048}
     for L, want in table.items():
         assert default_chunk_size(L) == want

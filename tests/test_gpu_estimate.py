@@ -102,3 +102,49 @@ def test_workspace_limit_splits_the_launch_without_changing_results(monkeypatch)
     monkeypatch.setattr(X, "WORKSPACE_LIMIT", 1 << 20)     # forces several chunk groups
     b = X.estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, causal=True, want_lists=False)["sums"]
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("mode", ["slash", "random", "double", "triple"])
+@pytest.mark.parametrize("S,C,L", [(8, 512, 1300), (16, 1024, 2048), (4, 256, 1024)])
+def test_select_modes_match_oracle(S, C, L, mode, causal):
+    """The other reshapes of the reference's torch branch (xattn/src/Xattention.py:72-135)
+    through the public operator: block sums against the oracle (fp32 inputs, so
+    its rolled key sums are exact like the kernel's fp32 accumulation)."""
+    from xattn.src.Xattention import xattn_estimate
+
+    q, k = _mk(4, 2, L, L, 20 + S)
+    torch.manual_seed(123)                 # "random" draws torch.randperm(stride) from the global generator
+    perm = torch.randperm(S)
+    torch.manual_seed(123)
+    got, mask = xattn_estimate(q.cuda(), k.cuda(), 128, S, threshold=0.9, chunk_size=C, select_mode=mode,
+                               causal=causal)
+    want, want_mask = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, S, threshold=0.9,
+                                       chunk_size=C, select_mode=mode, causal=causal, pad0_quirk=False, perm=perm)
+    assert got.shape == want.shape and got.dtype == torch.bfloat16
+    assert torch.allclose(got.float().cpu(), want, rtol=1e-2, atol=1e-3)     # bf16 result of the public operator
+    assert (mask.cpu() != want_mask).float().mean().item() < 5e-3
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_softmax_false_matches_oracle(causal):
+    """softmax=False (xattn/src/Xattention.py:231-234): block sums of exp(scaled score)."""
+    from xattn.src.Xattention import estimate_and_select
+
+    S, C, L = 8, 512, 1300
+    q, k = _mk(4, 2, L, L, 31, scale=1.5)
+    r = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=causal, want_lists=False, softmax=False)
+    want, _ = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, S, threshold=0.9, chunk_size=C,
+                               causal=causal, pad0_quirk=False, softmax=False)
+    assert torch.allclose(r["sums"].cpu(), want[0], rtol=2e-4, atol=2e-5)
+
+
+def test_bad_slab_pairs_are_refused():
+    from xattn.src import hip_backend as hb
+    from xattn.src.Xattention import estimate_and_select
+
+    q, k = _mk(2, 2, 512, 512, 1)
+    with pytest.raises(hb.XattnHipError):
+        estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, slab_pairs=[(8, 0)])      # offset outside the stride
+    with pytest.raises(hb.XattnHipError):
+        estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, slab_pairs=[(0, 0)] * 65)  # more than 64 pairs

@@ -52,3 +52,34 @@ def test_a_transposed_or_unreversed_operand_would_fail():
     ).transpose(2, 3)
     assert not torch.allclose(unreversed, good, atol=1e-6)
     assert torch.allclose(O.antidiagonal_scores(q, k, S), good, atol=1e-10)
+
+
+@pytest.mark.parametrize("mode", ["slash", "random", "double", "triple"])
+@pytest.mark.parametrize("S", [4, 8])
+def test_select_modes_are_sums_over_offset_pairs(mode, S):
+    """Every select_mode of the torch branch (xattn/src/Xattention.py:72-135) is a
+    sum of Q[m*S + a] . K[n*S + b] over a fixed list of (a, b): the lists below
+    are written out by hand, independently of the product's table."""
+    g = torch.Generator().manual_seed(S)
+    q = torch.randn(1, 2, 5 * S, 8, generator=g, dtype=torch.float64)
+    k = torch.randn(1, 2, 7 * S, 8, generator=g, dtype=torch.float64)
+    perm = torch.randperm(S, generator=g)
+    rq, rk = O.reshape_operands(q, k, S, mode, perm)
+    got = rq @ rk.transpose(2, 3)
+    full = torch.einsum("bhqd,bhkd->bhqk", q, k)
+    pairs = {
+        "slash": [(i, i, 1) for i in range(S)],
+        "random": [(int(perm[i]), i, 1) for i in range(S)],
+        "double": [(S - 1 - i, i, 1) for i in range(S)] + [(S - 1 - i, (i + 1) % S, 1) for i in range(S)],
+        "triple": [(S - 1 - i, i, 2) for i in range(S)] + [(S - 1 - i, (i + 1) % S, 1) for i in range(S)]
+        + [(S - 1 - i, (i - 1) % S, 1) for i in range(S)],
+    }[mode]
+    want = sum(w * full[:, :, a::S, b::S] for a, b, w in pairs)
+    assert torch.allclose(got, want, atol=1e-10)
+    # and the product's table encodes the same list
+    from xattn.src.Xattention import slab_pairs_for
+    import collections
+
+    table = collections.Counter(slab_pairs_for(mode, S, perm))
+    assert table == collections.Counter({(a, b): w for a, b, w in pairs})
+    assert slab_pairs_for("inverse", S) is None

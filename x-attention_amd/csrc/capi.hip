@@ -13,7 +13,7 @@ __global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* __re
 }
 }  // namespace xattn
 
-extern "C" int xattn_abi_version(void) { return 1; }
+extern "C" int xattn_abi_version(void) { return 2; }
 
 extern "C" const char* xattn_error_string(int code) {
   switch (code) {

@@ -47,7 +47,13 @@ struct EstParams {
   int off;                  // n_rk - n_rq: position of query row 0 on the key axis
   int real_rows;            // query rows >= real_rows are padding
   int causal, own_chunk_only;
+  int no_softmax;           // block sums of exp(scaled score) instead of softmax probabilities
   float scale_log2;
+  // Depth slabs of the reshaped GEMM.  Slab j multiplies query token
+  // m*S + (pairs[j] >> 4) with key token n*S + (pairs[j] & 15); n_pairs = 0 means
+  // the S pairs (S-1-i, i) of the antidiagonal reshape, in closed form.
+  int n_pairs;
+  uint8_t pairs[64];
   int nMT, nNT;             // tile rows over [row_begin, row_end) / tile columns over n_rk
   int tiles_per_head;       // tiles with a visible pair, per head
   int64_t total_tiles;      // tiles_per_head * H
@@ -183,12 +189,18 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   // before the LAST sub-step's MFMAs: at that point every fragment of the
   // current stage has been read, so the sub-step can prefetch the next stage's
   // first fragments and start refilling the current stage while its MFMAs run.
-  const int steps = p.S * 2;
+  const int steps = (p.n_pairs ? p.n_pairs : p.S) * 2;
   int voffK[4], voffQ[4];
   slab_offsets(k_snb, p.S, lane, wave, voffK);
   slab_offsets(q_snb, p.S, lane, wave, voffQ);
-  auto step_off_k = [&](int t) { return (t >> 1) * (int)k_snb + (t & 1) * kDepth * 2; };
-  auto step_off_q = [&](int t) { return (p.S - 1 - (t >> 1)) * (int)q_snb + (t & 1) * kDepth * 2; };
+  auto step_off_k = [&](int t) {
+    const int i = p.n_pairs ? (p.pairs[t >> 1] & 15) : (t >> 1);
+    return i * (int)k_snb + (t & 1) * kDepth * 2;
+  };
+  auto step_off_q = [&](int t) {
+    const int i = p.n_pairs ? (p.pairs[t >> 1] >> 4) : (p.S - 1 - (t >> 1));
+    return i * (int)q_snb + (t & 1) * kDepth * 2;
+  };
   // copy j (0..7) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
   auto copy_j = [&](int j, int t, char* stage) {
     const int tc = t < steps ? t : steps - 1;       // past the end: a harmless repeat
@@ -386,8 +398,9 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
 #pragma unroll
       for (int w = 0; w < 4; ++w) Lr += redL[w][lane] * fast_exp2(redM[w][lane] - safe);
       const bool real = row_ok && mc < p.real_rows && Lr > 0.f;
-      rowM[lane] = safe;
-      rowInv[lane] = real ? 1.f / Lr : 0.f;
+      // without softmax the partial sums are referred to 2^0 and left unnormalised
+      rowM[lane] = p.no_softmax ? 0.f : safe;
+      rowInv[lane] = real ? (p.no_softmax ? 1.f : 1.f / Lr) : 0.f;
     }
     __syncthreads();
   }
@@ -486,7 +499,8 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
                                          int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                                          int64_t k_stride_n, int stride, int block_size, int chunk_size,
                                          int chunk_begin, int chunk_end, int causal, int own_chunk_only,
-                                         float scale, void* stream) {
+                                         float scale, const int32_t* slab_pairs, int num_slab_pairs,
+                                         int softmax, void* stream) {
   if (!q || !k || !block_sums || !workspace) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
@@ -517,6 +531,15 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.causal = causal ? 1 : 0;
   p.own_chunk_only = own_chunk_only ? 1 : 0;
   p.scale_log2 = scale * kLog2e;
+  p.no_softmax = softmax ? 0 : 1;
+  p.n_pairs = 0;
+  if (num_slab_pairs < 0 || num_slab_pairs > 64 || (num_slab_pairs > 0 && !slab_pairs)) return XATTN_ERR_SHAPE;
+  for (int j = 0; j < num_slab_pairs; ++j) {
+    const int qo = slab_pairs[2 * j], ko = slab_pairs[2 * j + 1];
+    if (qo < 0 || qo >= stride || ko < 0 || ko >= stride) return XATTN_ERR_SHAPE;
+    p.pairs[j] = (uint8_t)((qo << 4) | ko);
+  }
+  p.n_pairs = num_slab_pairs;
   p.scores = scores_out;
   p.sums = block_sums;
   if (workspace_size < workspace_bytes(num_heads, g, p.rows)) return XATTN_ERR_WORKSPACE;

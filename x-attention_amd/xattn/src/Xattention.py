@@ -61,6 +61,29 @@ def _check_qk(x, name):
     return x
 
 
+def slab_pairs_for(select_mode, stride, perm=None):
+    """(query offset, key offset) pairs of the reshape for a ``select_mode`` of
+    xattn/src/Xattention.py:72-135, or None for the default antidiagonal one.
+    A pair (a, b) adds ``Q[m*S + a] . K[n*S + b]`` to score[m, n]."""
+    S = stride
+    if select_mode in ("inverse", ""):
+        return None
+    if select_mode == "slash":
+        return [(i, i) for i in range(S)]
+    if select_mode == "random":
+        if perm is None:
+            perm = torch.randperm(S)
+        return [(int(perm[i]), i) for i in range(S)]
+    if select_mode == "double":
+        # key slab i becomes K_i + K_(i+1): each query offset meets two key offsets
+        return [(S - 1 - i, i) for i in range(S)] + [(S - 1 - i, (i + 1) % S) for i in range(S)]
+    if select_mode == "triple":
+        # ... then that sum plus its own right-rolled copy: K_(i-1) + 2 K_i + K_(i+1)
+        base = [(S - 1 - i, i) for i in range(S)]
+        return base + base + [(S - 1 - i, (i + 1) % S) for i in range(S)] + [(S - 1 - i, (i - 1) % S) for i in range(S)]
+    raise ValueError(f"unknown select_mode {select_mode!r}")
+
+
 def _tau_per_head(threshold, heads, device):
     """float, 0-d tensor or [H] tensor -> float64 [H] on device, rounded the way
     the reference rounds it (a tensor keeps its own precision, utils.py:91-92)."""
@@ -78,8 +101,14 @@ class _Plan:
     """Geometry, buffers and kernel launchers of one estimate -> select pass."""
 
     def __init__(self, query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, want_lists, dump_scores):
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs=None, softmax=True):
         self.lib = _hb.lib()
+        self.softmax = bool(softmax)
+        self.n_pairs = 0 if slab_pairs is None else len(slab_pairs)
+        self.pairs = None
+        if self.n_pairs:
+            flat = [int(v) for pr in slab_pairs for v in pr]
+            self.pairs = (_hb.c_i32 * len(flat))(*flat)
         q = _check_qk(query_states, "query_states")
         k = _check_qk(key_states, "key_states")
         if k.device != q.device:
@@ -144,7 +173,8 @@ class _Plan:
                 self.heads, self.kv_heads, self.q_len, self.k_len, 128,
                 q.stride(1), q.stride(2), k.stride(1), k.stride(2),
                 self.stride, self.block_size, self.chunk_size, chunk_begin, chunk_end,
-                int(self.causal), int(self.own_chunk_only), self.scale, stream,
+                int(self.causal), int(self.own_chunk_only), self.scale, self.pairs, self.n_pairs,
+                int(self.softmax), stream,
             ),
             "xattn_estimate_block_sums",
         )
@@ -182,6 +212,8 @@ def estimate_and_select(
     want_lists=True,
     dump_scores=False,
     marks=None,
+    slab_pairs=None,
+    softmax=True,
 ):
     """Runs the estimator and selection kernels over all query chunks, one launch each.
 
@@ -194,7 +226,7 @@ def estimate_and_select(
     and after selection (for per-kernel timing).
     """
     plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, want_lists, dump_scores)
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs, softmax)
     with torch.cuda.device(plan.dev):
         stream = _stream_ptr(plan.dev)
         _mark(marks, "estimate_begin")
@@ -226,19 +258,18 @@ def xattn_estimate(
     Same contract as xattn/src/Xattention.py:13-299: returns
     ``(attn_sums, simple_masks)``, both ``[1, H, Nq_p, Nk_p]`` over the lengths
     padded to multiples of ``chunk_size``; ``attn_sums`` in the query dtype,
-    ``simple_masks`` bool.  Only ``select_mode="inverse"``, ``kdb=1`` and
-    ``softmax=True`` (what every caller in the reference uses) are implemented.
+    ``simple_masks`` bool.  ``select_mode`` ("inverse", "slash", "random",
+    "double", "triple"; the reference has the last four in its torch branch only,
+    Xattention.py:72-135) and ``softmax=False`` (:231-234) run on the same
+    kernel; "random" draws ``torch.randperm(stride)`` like the reference.
+    ``kdb != 1`` (query rows subsampled, no caller uses it) is not provided.
     """
-    if select_mode not in ("inverse", ""):
-        raise NotImplementedError(f"select_mode={select_mode!r} is not implemented on the HIP path")
     if kdb != 1:
         raise ValueError("kdb != 1 is not supported by the fused estimator")
-    if not softmax:
-        raise NotImplementedError("softmax=False is not implemented on the HIP path")
     r = estimate_and_select(
         query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
         use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
-        want_lists=False,
+        want_lists=False, slab_pairs=slab_pairs_for(select_mode, stride), softmax=softmax,
     )
     attn_sums = r["sums"].to(query_states.dtype).unsqueeze(0)
     simple_masks = r["mask"].view(torch.bool).unsqueeze(0)
