@@ -176,6 +176,21 @@ int xattn_decode_fwd(const void* q, const void* k, const void* v, void* out, voi
                      int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Stand-alone softmax + block sums over a score matrix in memory: the seam
+ * softmax_fuse_block_sum, xattn/src/kernels.py:238-289 (kernels :5-156), for
+ * callers that hold the strided scores themselves (the fused estimator above
+ * does not use it).  `scores` is bf16 [num_heads][n_rq][n_rk] with head / row
+ * strides in elements (multiples of 8, rows contiguous); row i sits at key
+ * position chunk_start + i.  p = exp2(score * scale - rowmax) / rowsum over the
+ * visible keys (causal != 0: keys <= chunk_start + i; else all n_rk), rows at
+ * positions >= real_q_len give zeros; block_sums is fp32
+ * [num_heads][n_rq / rbs][n_rk / rbs], rbs = reshaped_block_size in {8, 16, 32}.
+ */
+int xattn_softmax_block_sums(const void* scores, float* block_sums, int num_heads, int n_rq, int n_rk,
+                             int64_t stride_h, int64_t stride_row, int reshaped_block_size, int chunk_start,
+                             int real_q_len, float scale, int causal, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Threshold profiler, xattn/threshold/profile_threshold/profile_threshold.py.
  *
  * xattn_block_mass replaces chunk_prefill_to_attn_sum (:15-57): the true

@@ -90,8 +90,40 @@ def test_seam_flat_group_gemm_fuse_reshape(is_causal):
     assert out.shape == (1, 2, 128, 384) and out.dtype == torch.bfloat16
     cols = 256 if is_causal else 384            # tiles past the chunk's diagonal are not computed
     assert torch.allclose(out[..., :cols].float().cpu(), want[..., :cols], rtol=1e-2, atol=0.2)
-    with pytest.raises(NotImplementedError):
-        softmax_fuse_block_sum(out, 16, 16, 128, 256, 384, 1.0)
+    # ... and the second seam on those very scores, the reference's own two-step sequence
+    # (xattn/src/Xattention.py:141-172), against a plain torch softmax of them
+    scale = 1.4426950408889634 / math.sqrt(128) / S
+    sums = softmax_fuse_block_sum(out, 16, 16, 128, 256, 300, scale, is_causal=is_causal)
+    assert sums.shape == (1, 2, 8, 24) and sums.dtype == torch.bfloat16
+    x = out.float().cpu() * (scale / 1.4426950408889634)
+    if is_causal:
+        pos = torch.arange(128)[:, None] + 128
+        x = x.masked_fill(torch.arange(384)[None, :] > pos, float("-inf"))
+    p = torch.softmax(x, -1)
+    p[:, :, 300 - 128:, :] = 0                      # rows at positions >= real_q_len
+    want_sums = p.view(1, 2, 8, 16, 24, 16).sum(-1).sum(-2)
+    assert torch.allclose(sums.float().cpu(), want_sums, rtol=1e-2, atol=1e-3)
+
+
+@pytest.mark.parametrize("rbs,n_rq,n_rk,start", [(8, 64, 1024, 960), (32, 96, 2048, 512), (16, 16, 528, 0)])
+def test_seam_softmax_fuse_block_sum_fp32_check(rbs, n_rq, n_rk, start):
+    """Closer check of the stand-alone kernel through the C ABI (fp32 output)."""
+    from xattn.src import hip_backend as hb
+
+    g = torch.Generator().manual_seed(rbs)
+    x = (3.0 * torch.randn(3, n_rq, n_rk, generator=g)).bfloat16()
+    xd = x.cuda()
+    for causal in (1, 0):
+        out = torch.empty(3, n_rq // rbs, n_rk // rbs, dtype=torch.float32, device="cuda")
+        hb.check(hb.lib().xattn_softmax_block_sums(xd.data_ptr(), out.data_ptr(), 3, n_rq, n_rk, xd.stride(0),
+                                                   xd.stride(1), rbs, start, start + n_rq - 5, 0.7, causal, None), "sbs")
+        s = x.double() * 0.7 * math.log(2.0)
+        if causal:
+            s = s.masked_fill(torch.arange(n_rk)[None, :] > torch.arange(n_rq)[:, None] + start, float("-inf"))
+        p = torch.softmax(s, -1)
+        p[:, n_rq - 5:] = 0
+        want = p.view(3, n_rq // rbs, rbs, n_rk // rbs, rbs).sum(-1).sum(-2)
+        assert torch.allclose(out.double().cpu(), want, rtol=1e-4, atol=1e-6), (causal, (out.double().cpu() - want).abs().max())
 
 
 def test_workspace_limit_splits_the_launch_without_changing_results(monkeypatch):

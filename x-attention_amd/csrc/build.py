@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-SOURCES = ["capi.hip", "block_sparse_attn.hip", "estimate.hip", "select_blocks.hip", "decode_attn.hip", "profile_threshold.hip"]
+SOURCES = ["capi.hip", "block_sparse_attn.hip", "estimate.hip", "select_blocks.hip", "decode_attn.hip", "profile_threshold.hip", "softmax_block_sum.hip"]
 LIB = os.path.join(HERE, "libxattn_hip.so")
 FLAGS = [
     "--offload-arch=gfx950",

@@ -3,10 +3,10 @@ seams over the fused HIP estimator.
 
 The reference runs two Triton kernels back to back - the strided-reshape GEMM
 and the softmax / block-sum pass over the score matrix it wrote.  Here both
-live in one estimator that never materialises the scores, so only the first
-name has a stand-alone meaning: it asks the estimator to also dump its raw
-scores (a debugging path).  ``softmax_fuse_block_sum`` on a caller-supplied
-score matrix is not provided; ``xattn_estimate`` returns the block sums.
+live in one estimator that never materialises the scores.  The two names are
+kept for callers that use them on their own: the first asks the estimator to
+dump its raw scores, the second runs a stand-alone softmax / block-sum kernel
+over a caller-supplied score matrix.  ``xattn_estimate`` uses neither.
 """
 import math
 
@@ -63,9 +63,44 @@ def flat_group_gemm_fuse_reshape(query_states, key_states, stride, chunk_start, 
     return out.to(query_states.dtype).unsqueeze(0)
 
 
-def softmax_fuse_block_sum(*args, **kwargs):
-    """Not available as a separate pass: the estimator fuses it (see
-    ``xattn.src.Xattention.xattn_estimate``, which returns the block sums)."""
-    raise NotImplementedError(
-        "softmax_fuse_block_sum is fused into the HIP estimator; call xattn_estimate for the block sums"
-    )
+def softmax_fuse_block_sum(attn_weights_slice, reshaped_block_size, segment_size, chunk_start, chunk_end,
+                           real_q_len, scale, is_causal=True):
+    """Row softmax of a score matrix and its sums over
+    ``reshaped_block_size`` x ``reshaped_block_size`` tiles.
+
+    Same contract as xattn/src/kernels.py:238-289: ``attn_weights_slice`` is
+    ``[1, H, q_r, k_r]`` raw scores of a query chunk whose row 0 sits at key
+    position ``chunk_start``; ``scale`` multiplies them and already contains
+    log2(e) (the softmax is taken with exp2); with ``is_causal`` row ``i`` sees
+    keys ``<= chunk_start + i``; rows at positions ``>= real_q_len`` come out as
+    zeros.  Returns ``[1, H, q_r / rbs, k_r / rbs]`` in the input dtype.
+    ``segment_size`` only sets the reference kernel's inner tile; it is checked
+    and otherwise unused.  The fused estimator does not go through here.
+    """
+    lib = _hb.lib()
+    x = attn_weights_slice
+    if not x.is_cuda:
+        raise _hb.XattnHipError("attn_weights_slice must live on a ROCm device (no CPU fallback exists)")
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"attn_weights_slice must be torch.bfloat16, got {x.dtype}")
+    batch_size, num_heads, q_len, k_len = x.shape
+    assert batch_size == 1
+    assert q_len % reshaped_block_size == 0
+    assert k_len % segment_size == 0
+    assert segment_size % reshaped_block_size == 0
+    assert x.stride(-1) == 1
+    assert chunk_end - chunk_start == q_len
+    if x.stride(1) % 8 or x.stride(2) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    with torch.cuda.device(x.device):
+        out = torch.empty((1, num_heads, q_len // reshaped_block_size, k_len // reshaped_block_size),
+                          dtype=torch.float32, device=x.device)
+        _hb.check(
+            lib.xattn_softmax_block_sums(
+                x.data_ptr(), out.data_ptr(), num_heads, q_len, k_len, x.stride(1), x.stride(2),
+                reshaped_block_size, chunk_start, real_q_len, float(scale), int(bool(is_causal)),
+                _stream_ptr(x.device),
+            ),
+            "xattn_softmax_block_sums",
+        )
+    return out.to(attn_weights_slice.dtype)
