@@ -104,7 +104,8 @@ __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk
 
 
 // kDump: also write the raw scores (test / seam builds only; kept out of the production instantiation)
-template <int RBS, bool kDump>
+// kTable: the depth slabs come from p.pairs (the non-default select modes); the default keeps its closed form
+template <int RBS, bool kDump, bool kTable>
 __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -189,16 +190,16 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   // before the LAST sub-step's MFMAs: at that point every fragment of the
   // current stage has been read, so the sub-step can prefetch the next stage's
   // first fragments and start refilling the current stage while its MFMAs run.
-  const int steps = (p.n_pairs ? p.n_pairs : p.S) * 2;
+  const int steps = (kTable ? p.n_pairs : p.S) * 2;
   int voffK[4], voffQ[4];
   slab_offsets(k_snb, p.S, lane, wave, voffK);
   slab_offsets(q_snb, p.S, lane, wave, voffQ);
   auto step_off_k = [&](int t) {
-    const int i = p.n_pairs ? (p.pairs[t >> 1] & 15) : (t >> 1);
+    const int i = kTable ? (p.pairs[t >> 1] & 15) : (t >> 1);
     return i * (int)k_snb + (t & 1) * kDepth * 2;
   };
   auto step_off_q = [&](int t) {
-    const int i = p.n_pairs ? (p.pairs[t >> 1] >> 4) : (p.S - 1 - (t >> 1));
+    const int i = kTable ? (p.pairs[t >> 1] >> 4) : (p.S - 1 - (t >> 1));
     return i * (int)q_snb + (t & 1) * kDepth * 2;
   };
   // copy j (0..7) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
@@ -449,7 +450,8 @@ using namespace xattn;
 namespace {
 template <int RBS>
 hipError_t launch_gemm(const EstParams& p, dim3 grid, size_t lds, hipStream_t s) {
-  auto kernel = p.scores ? &estimate_gemm_kernel<RBS, true> : &estimate_gemm_kernel<RBS, false>;
+  auto kernel = p.n_pairs ? (p.scores ? &estimate_gemm_kernel<RBS, true, true> : &estimate_gemm_kernel<RBS, false, true>)
+                          : (p.scores ? &estimate_gemm_kernel<RBS, true, false> : &estimate_gemm_kernel<RBS, false, false>);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return e;
