@@ -28,7 +28,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs whose summary is
 # kept under profiles/ (counters cannot be read from inside this process); other workloads report null.
-MEASURED_TRAFFIC_BYTES = {"cfg2_llama8b_L131072_gqa32x8_S16": 2.024e10}
+MEASURED_TRAFFIC_BYTES = {"cfg2_llama8b_L131072_gqa32x8_S16": 6.33e9}
 
 
 def _ms(a, b):
