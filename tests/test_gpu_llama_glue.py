@@ -51,6 +51,26 @@ def test_full_metric_prefill_and_decode_match_stock_attention():
             nxt = a.logits[:, -1:].argmax(-1)
 
 
+def test_static_cache_is_cut_to_its_filled_part():
+    from transformers import StaticCache
+    from xattn.src.load_llama import FastPrefillConfig, patch_model
+
+    stock = _tiny_llama(5)
+    ours = patch_model(copy.deepcopy(stock), FastPrefillConfig(threshold=0.9, metric="full"))
+    ids = torch.randint(0, 512, (1, 700), generator=torch.Generator().manual_seed(6)).cuda()
+    with torch.no_grad():
+        a = stock(ids, use_cache=True)                              # growing cache
+        cache = StaticCache(config=ours.config, max_cache_len=1024)
+        b = ours(ids, past_key_values=cache, use_cache=True)        # preallocated cache, 1024 slots
+        assert _rel(b.logits, a.logits) < 3e-2
+        nxt = a.logits[:, -1:].argmax(-1)
+        for _ in range(2):
+            a = stock(nxt, past_key_values=a.past_key_values, use_cache=True)
+            b = ours(nxt, past_key_values=cache, use_cache=True)
+            assert _rel(b.logits, a.logits) < 3e-2
+            nxt = a.logits[:, -1:].argmax(-1)
+
+
 def test_xattn_metric_calls_match_oracle(monkeypatch):
     from xattn.src import load_llama
     from xattn.src.load_llama import FastPrefillConfig, patch_model

@@ -86,6 +86,14 @@ class FastPrefillConfig(dict):
         return self.threshold
 
 
+def _is_static_cache(cache):
+    try:
+        from transformers import StaticCache
+    except ImportError:
+        return False
+    return isinstance(cache, StaticCache)
+
+
 def _stamp(cfg, label, start):
     if cfg.print_detail:
         torch.cuda.synchronize()
@@ -129,9 +137,13 @@ def forward_eval(self, hidden_states, position_embeddings=None, attention_mask=N
     if cache is not None:
         cache_kwargs = {"sin": sin, "cos": cos, "cache_position": cache_position}
         key_states, value_states = cache.update(key_states, value_states, self.layer_idx, cache_kwargs)
-        if cache_position is not None and key_states.shape[2] > q_len:
-            # a preallocated cache hands back its whole buffer: keep what is filled (load_llama.py:152-154)
-            filled = min(int(cache_position[-1]) + 1, key_states.shape[2])
+        if _is_static_cache(cache):
+            # a preallocated cache hands back its whole buffer: keep what is filled (load_llama.py:152-154).
+            # The last position comes from cache_position where the model code passes it, else from position_ids.
+            pos = cache_position if cache_position is not None else (position_ids[0] if position_ids is not None else None)
+            if pos is None:
+                raise ValueError("a static cache needs cache_position or position_ids to know how much of it is filled")
+            filled = min(int(pos[-1]) + 1, key_states.shape[2])
             key_states, value_states = key_states[:, :, :filled], value_states[:, :, :filled]
     if key_states.device != query_states.device:
         key_states = key_states.to(query_states.device)
