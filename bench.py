@@ -127,6 +127,37 @@ def decode_leg(q, k, v, reps=50):
     }
 
 
+def mfma_probe(dev):
+    """What a stream of bf16 MFMAs alone sustains on this part: with constant operand bits and with
+    random ones (the clock the part holds depends on the switching activity of the operands)."""
+    import ctypes
+
+    import torch
+    from xattn.src import hip_backend
+
+    lib = hip_backend.lib()
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    res = {}
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    tables = {
+        "constant_operands": torch.full((4096 * 8,), 0.5, dtype=torch.bfloat16),
+        "random_operands": torch.randn(4096 * 8, generator=gen).bfloat16(),
+    }
+    for name, host in tables.items():
+        bits = host.to(dev)
+        flops = ctypes.c_double(0.0)
+        stream = torch.cuda.current_stream().cuda_stream
+        hip_backend.check(lib.xattn_mfma_rate_probe(bits.data_ptr(), 20000, sink.data_ptr(), ctypes.byref(flops), stream), "probe")
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        hip_backend.check(lib.xattn_mfma_rate_probe(bits.data_ptr(), 100000, sink.data_ptr(), ctypes.byref(flops), stream), "probe")
+        e1.record()
+        torch.cuda.synchronize()
+        res[name + "_tflops"] = round(flops.value / (_ms(e0, e1) * 1e-3) / 1e12, 1)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,6 +167,7 @@ def main():
     ap.add_argument("--dense-steps", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode-step measurement")
+    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only rate probe")
     ap.add_argument("--compare-pipelined", action="store_true",
                     help="also time Xattention_prefill with and without chunk-by-chunk stream pipelining")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -287,6 +319,8 @@ def main():
         del src, dst
     if not args.no_decode:
         result["decode_step"] = decode_leg(q, k, v)
+    if not args.no_mfma_probe:
+        result["mfma_alone"] = mfma_probe(dev)
     if not args.no_cpu_baseline:
         base, (cq, ck, cv, cmask) = cpu_baseline()
         # the same sample on the GPU path (bf16), for scale

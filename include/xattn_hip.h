@@ -228,6 +228,18 @@ int xattn_threshold_rows(const float* block_mass, const float* estimate_sums, fl
  */
 int xattn_calibration_copy(void* dst, const void* src, size_t bytes, void* stream);
 
+/* Measurement aid, no counterpart in the reference: 512 workgroups (two
+ * wavefronts per SIMD on 256 CUs) issue nothing but bf16 32x32x16 MFMAs,
+ * 16 * iters per wavefront, on register operands taken once from
+ * `operand_bits` (device, 64 KiB: 4096 fragments of 8 bf16).  The number of
+ * floating-point operations of the launch is written to *flops_out (host, may
+ * be null); the caller times the launch.  Equal bits everywhere measure the
+ * data-independent rate, random bits the rate the part sustains at the
+ * switching activity of real inputs.  `sink` is one float of device memory that
+ * is practically never written.
+ */
+int xattn_mfma_rate_probe(const void* operand_bits, int iters, float* sink, double* flops_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,6 +11,42 @@ __global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* __re
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
     dst[i] = src[i];
 }
+
+// Nothing but bf16 32x32x16 MFMAs on register operands: what the matrix pipes
+// sustain with no memory, LDS or VALU work beside them.  The operands are 16
+// fragments per lane read once from `bits` (4 KiB-entries table of 16-byte
+// fragments): all-equal bits give the data-independent rate, random bits the
+// rate at the switching activity of real inputs - the clock the part holds
+// differs between the two.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 probe_bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float probe_f32x16;
+__global__ __launch_bounds__(256) void mfma_rate_probe_kernel(const probe_bf16x8* __restrict__ bits, int iters,
+                                                              float* sink) {
+  probe_bf16x8 a[8], b[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    a[e] = bits[(threadIdx.x * 16 + e) & 4095];
+    b[e] = bits[(threadIdx.x * 16 + 8 + e) & 4095];
+  }
+  probe_f32x16 acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(u * 4 + i) & 7], b[(u + i) & 7], acc[i], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s += acc[i][v];
+  if (s == 12345.678f) sink[0] = s;   // keeps the accumulators live; practically never taken
+}
 }  // namespace xattn
 
 extern "C" int xattn_abi_version(void) { return 2; }
@@ -37,5 +73,17 @@ extern "C" int xattn_calibration_copy(void* dst, const void* src, size_t bytes, 
   hipLaunchKernelGGL(xattn::calibration_copy_kernel, dim3(256 * 32), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint4*>(src),
                      static_cast<uint4*>(dst), bytes / 16);
+  return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
+}
+
+extern "C" int xattn_mfma_rate_probe(const void* operand_bits, int iters, float* sink, double* flops_out,
+                                     void* stream) {
+  if (!operand_bits || !sink) return XATTN_ERR_NULL;
+  if (iters <= 0 || iters > (1 << 22)) return XATTN_ERR_SHAPE;
+  if (reinterpret_cast<uintptr_t>(operand_bits) & 15) return XATTN_ERR_ALIGN;
+  const int grid = 256 * 2;   // two workgroups of four wavefronts per CU: two wavefronts per SIMD
+  if (flops_out) *flops_out = (double)grid * 4.0 * iters * 16.0 * 32768.0;
+  hipLaunchKernelGGL(xattn::mfma_rate_probe_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const xattn::probe_bf16x8*>(operand_bits), iters, sink);
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
 }
