@@ -47,6 +47,31 @@ def test_host_side_calls_need_no_gpu():
     assert lib.xattn_estimate_workspace_bytes(32, 4096, 2048, 8, 128, 2048, 0) == 0          # k shorter than q
 
 
+def test_attention_entry_points_validate_strides_and_scale_before_launching():
+    """Host-side validation only: the calls return before anything is enqueued,
+    so dummy (aligned, non-null) addresses are enough."""
+    from xattn.src import hip_backend as hb
+
+    lib = hb.lib()
+    a = 0x10000
+    ok_strides = [128 * 256, 128, 128 * 256, 128, 128 * 256, 128, 128, 128 * 4]
+
+    def fwd(strides, scale=0.1, heads=4, kv=2):
+        return lib.xattn_block_sparse_fwd(a, a, a, a, None, None, 0, 0, heads, kv, 256, 256, 128, *strides, 0, -1, 1,
+                                          scale, None)
+
+    big = 1 << 23
+    assert fwd([ok_strides[0], 128, ok_strides[2], big] + ok_strides[4:]) == -4        # K token stride beyond 2^22
+    assert fwd(ok_strides[:5] + [big] + ok_strides[6:]) == -4                          # V token stride
+    assert fwd(ok_strides[:3] + [64] + ok_strides[4:]) == -4                           # rows would overlap
+    assert fwd(ok_strides, scale=0.0) == -4 and fwd(ok_strides, scale=-1.0) == -4
+    assert fwd(ok_strides, scale=float("nan")) == -4
+    assert fwd(ok_strides, heads=3, kv=2) == -3
+    mass = lambda ksn, scale=0.1: lib.xattn_block_mass(a, a, a, 4, 2, 256, 256, 128, 128 * 256, 128, 128 * 256, ksn, 1,
+                                                       scale, None)
+    assert mass(big) == -4 and mass(64) == -4 and mass(128, scale=0.0) == -4
+
+
 def test_operator_refuses_cpu_tensors_and_wrong_dtypes():
     import torch
 

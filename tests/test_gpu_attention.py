@@ -76,6 +76,19 @@ def test_strided_views_and_gqa_equal_repeated_kv():
     _check(a, want)
 
 
+@pytest.mark.parametrize("H,Hkv", [(71, 1), (128, 1), (130, 2)])
+def test_more_than_64_query_heads_per_kv_head(H, Hkv):
+    """A KV head's query heads are dispatched in sets of at most 64: every head is computed."""
+    from xattn.src.Xattention import block_sparse_attention
+
+    L = 300
+    q, k, v = _mk(H, Hkv, L, L, 7)
+    out = torch.full((1, L, H, 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    got = block_sparse_attention(q.cuda(), k.cuda(), v.cuda(), causal=True, out=out)
+    want = O.block_sparse_attention(q, k, v, torch.ones(1, H, 3, 3, dtype=torch.bool), causal=True)
+    _check(got, want)
+
+
 def test_rejects_bad_arguments():
     from xattn.src import hip_backend as hb
     from xattn.src.Xattention import block_sparse_attention

@@ -1,0 +1,82 @@
+"""GPU: block-mask parity with the oracle AT the benchmark's sizes.
+
+For every GPU workload (and, where the key length is a multiple of the chunk
+size, both settings of ``use_triton``) the estimate and selection run for all
+heads on the HIP path; the oracle then runs on the host, in fp32, for the query
+heads with the fewest and the most kept blocks, on the very bf16 values the
+kernels read.  Masks must agree except for blocks whose decision sits within
+1e-5 of the threshold; those are counted and printed.  Workload 0 (the CPU
+configuration) is run on its bf16 cast for all 32 heads.
+"""
+import pytest
+import torch
+
+from helpers import head_mask_parity
+
+pytestmark = pytest.mark.gpu
+
+SUMS_ATOL = 2e-5
+SUMS_RTOL = 2e-4
+
+
+def _check_heads(w, q, k, r, heads, chunk, use_triton):
+    tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "outside_band": 0}
+    for h in heads:
+        rep = head_mask_parity(q, k, h, r["mask"][h], w.stride, w.threshold, chunk, w.causal,
+                               pad0_quirk=not use_triton, sums_got=r["sums"][h])
+        print(f"{w.name} use_triton={use_triton} {rep}", flush=True)
+        for key in tot:
+            tot[key] += rep[key]
+        assert rep["outside_band"] == 0, rep
+        # block sums of a row add up to block_size / stride: the absolute tolerance is relative to that
+        assert rep["sums_max_abs_diff"] <= SUMS_ATOL + SUMS_RTOL * (128 // w.stride), rep
+    return tot
+
+
+@pytest.mark.parametrize("idx,use_triton", [(1, True), (1, False), (2, True), (2, False), (3, True), (3, False), (4, True)])
+def test_mask_parity_at_benchmark_size(idx, use_triton):
+    from xattn.src.Xattention import default_chunk_size, estimate_and_select
+    from xattn.synthetic import WORKLOADS, make_inputs
+
+    w = WORKLOADS[idx]
+    q, k, _ = make_inputs(w, device="cuda", seed=0)
+    chunk = w.chunk_size or default_chunk_size(w.L)
+    r = estimate_and_select(q, k, w.stride, w.threshold, chunk, causal=w.causal, use_triton=use_triton)
+    torch.cuda.synchronize()
+    kept = r["col_cnt"].long().sum(-1)
+    heads = sorted({int(kept.argmin()), int(kept.argmax())})
+    if len(heads) == 1:
+        heads.append((heads[0] + 1) % w.heads)
+    tot = _check_heads(w, q, k, r, heads, chunk, use_triton)
+    print(f"{w.name} use_triton={use_triton}: heads {heads} total {tot}", flush=True)
+
+
+@pytest.mark.parametrize("use_triton", [True, False])
+def test_mask_parity_on_the_cpu_configuration(use_triton):
+    """Workload 0 (32 MHA heads, L=4096, stride 8, chunk 2048) on its bf16 cast, every head."""
+    from xattn.src.Xattention import estimate_and_select
+    from xattn.synthetic import WORKLOADS, make_inputs
+
+    w = WORKLOADS[0]
+    q, k, _ = make_inputs(w, device="cpu", seed=0)
+    q, k = q.bfloat16(), k.bfloat16()
+    r = estimate_and_select(q.cuda(), k.cuda(), w.stride, w.threshold, w.chunk_size, causal=True, use_triton=use_triton)
+    torch.cuda.synchronize()
+    tot = _check_heads(w, q, k, r, range(w.heads), w.chunk_size, use_triton)
+    assert tot["blocks"] == 32 * 32 * 32
+    print(f"{w.name} (bf16 cast) use_triton={use_triton}: total {tot}", flush=True)
+
+
+def test_sampled_rows_at_the_headline_size_with_a_small_workspace(monkeypatch):
+    """The grouped-launch path (estimator workspace bounded, several launches) at
+    L=131072 gives the very block sums and masks of the single launch."""
+    import xattn.src.Xattention as X
+    from xattn.synthetic import WORKLOADS, make_inputs
+
+    w = WORKLOADS[2]
+    q, k, _ = make_inputs(w, device="cuda", seed=0, heads=4, kv_heads=1)
+    a = X.estimate_and_select(q, k, w.stride, w.threshold, w.chunk_size, causal=True)
+    monkeypatch.setattr(X, "WORKSPACE_LIMIT", 48 << 20)      # two query chunks per launch
+    b = X.estimate_and_select(q, k, w.stride, w.threshold, w.chunk_size, causal=True)
+    assert torch.equal(a["sums"], b["sums"]) and torch.equal(a["mask"], b["mask"])
+    assert torch.equal(a["col_cnt"], b["col_cnt"])

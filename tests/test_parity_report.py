@@ -1,0 +1,76 @@
+"""CPU: the band report the mask-parity tests rely on must flag flips away from
+the threshold crossing and tolerate flips at it."""
+import torch
+
+from oracle import xattn_oracle as O
+from oracle.parity import TAU_BAND, head_mask_parity, mask_mismatch_report
+
+
+def _row_case(causal):
+    # one head, 4 q-block rows over 8 columns (k_len > q_len by 4 blocks when causal)
+    g = torch.Generator().manual_seed(3)
+    x = torch.rand(1, 4, 8, generator=g, dtype=torch.float64) + 0.05
+    off = 4
+    if causal:
+        x = x * (torch.arange(8)[None, :] <= torch.arange(4)[:, None] + off)
+    want = O.find_blocks_chunked(x[None].float(), off, 0.6, None, decoding=False, mode="prefill", causal=causal)[0]
+    if causal:
+        want &= torch.arange(8)[None, :] <= torch.arange(4)[:, None] + off
+    return x.float(), want, off
+
+
+def test_flip_far_from_the_crossing_is_outside_the_band():
+    for causal in (True, False):
+        x, want, off = _row_case(causal)
+        assert mask_mismatch_report(x, want, want, 0.6, causal, off) == (0, 0)
+        # the largest non-forced block of row 2 is kept long before the crossing: dropping it is a real error
+        row = x[0, 2].clone()
+        if causal:
+            row[0] = row[2 + off] = -1
+        j = int(row.argmax())
+        got = want.clone()
+        assert got[0, 2, j]
+        got[0, 2, j] = False
+        assert mask_mismatch_report(x, got, want, 0.6, causal, off) == (1, 1)
+        if causal:   # forced blocks and blocks beyond the diagonal are never excused
+            got = want.clone()
+            got[0, 1, 1 + off] = False
+            got[0, 0, 7] = True
+            assert mask_mismatch_report(x, got, want, 0.6, causal, off) == (2, 2)
+
+
+def test_flip_at_the_crossing_is_inside_the_band():
+    # non-causal row [4, 3, 2, 1] (total 10): mass before the third block is 7 -> with tau = 0.7 the decision
+    # "7 < 7" sits exactly on the threshold; a path that sees 6.9999999 keeps the block
+    x = torch.tensor([[[4.0, 3.0, 2.0, 1.0]]])
+    want = O.find_blocks_chunked(x[None], 0, 0.7, None, decoding=False, mode="prefill", causal=False)[0]
+    assert want[0, 0].tolist() == [True, True, False, False]
+    got = want.clone()
+    got[0, 0, 2] = True
+    assert mask_mismatch_report(x, got, want, 0.7, False, 0) == (1, 0)
+    got[0, 0, 3] = True                      # the last block is a full unit of mass past the crossing
+    assert mask_mismatch_report(x, got, want, 0.7, False, 0) == (2, 1)
+    # shifting the threshold by more than the band makes the same flip an error
+    tau = 0.7 - 3 * TAU_BAND
+    want2 = O.find_blocks_chunked(x[None], 0, tau, None, decoding=False, mode="prefill", causal=False)[0]
+    got2 = want2.clone()
+    got2[0, 0, 2] = True
+    assert mask_mismatch_report(x, got2, want2, tau, False, 0) == (1, 1)
+
+
+def test_head_mask_parity_runs_one_head_of_a_grouped_layout():
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, 4, 512, 128, generator=g).bfloat16()
+    k = torch.randn(1, 2, 512, 128, generator=g).bfloat16()
+    sums, mask = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, 8, threshold=0.9, chunk_size=256,
+                                  pad0_quirk=False)
+    for h in range(4):
+        rep = head_mask_parity(q, k, h, mask[0, h], 8, 0.9, 256, True, False, sums_got=sums[0, h])
+        assert rep["mismatches"] == 0 and rep["blocks"] == 16 and rep["sums_max_abs_diff"] < 1e-5
+    wrong = mask[0, 3].clone()
+    wrong[3, 3] = False                       # a forced diagonal block
+    assert head_mask_parity(q, k, 3, wrong, 8, 0.9, 256, True, False)["outside_band"] == 1
+    taus = torch.tensor([0.5, 0.9, 0.7, 0.99])
+    _, m2 = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, 8, threshold=taus, chunk_size=256,
+                             pad0_quirk=False)
+    assert head_mask_parity(q, k, 2, m2[0, 2], 8, taus, 256, True, False)["mismatches"] == 0

@@ -47,34 +47,54 @@ __device__ __forceinline__ void tile_offsets(int64_t sn, int lane, int wave, int
 // workgroups each, one L2) starts its workgroups in id order.  The 64 ids that
 // land on one XCD one after the other form a unit: the query heads of ONE KV
 // head times a run of adjacent q-blocks, so everything resident on the XCD
-// streams the same K/V through its L2 at about the same place.  Units are
-// dealt to XCDs in turn; the KV head of a unit rotates with the q-block run,
-// so every XCD sees every head equally often (heads differ by orders of
-// magnitude in list length).  Runs go out last (longest, when causal) first.
+// streams the same K/V through its L2 at about the same place.  A KV head with
+// more than 64 query heads is dealt as several head sets of equal size (each a
+// dispatch group of its own).  Units are dealt to XCDs in turn; the dispatch
+// group of a unit rotates with the q-block run, so every XCD sees every head
+// equally often (heads differ by orders of magnitude in list length).  Runs go
+// out last (longest, when causal) first.
+struct DispatchShape {
+  int group;       // query heads per KV head
+  int sets;        // head sets per KV head (1 unless group > kUnit)
+  int set_heads;   // query heads per set (<= kUnit)
+  int n_groups;    // dispatch groups: Hkv * sets
+  int unit_rows;   // q-blocks per unit
+};
+__host__ __device__ inline DispatchShape dispatch_shape(int H, int Hkv) {
+  DispatchShape d;
+  d.group = H / Hkv;
+  d.sets = (d.group + kUnit - 1) / kUnit;
+  d.set_heads = (d.group + d.sets - 1) / d.sets;
+  d.n_groups = Hkv * d.sets;
+  d.unit_rows = kUnit / d.set_heads;
+  return d;
+}
+
 // Returns false for ids that carry no work.
-__device__ __forceinline__ bool map_workgroup(int id, int H, int Hkv, int unit_rows, int qb_begin, int qb_end,
-                                              int* head, int* qb) {
-  const int group = H / Hkv;
+__host__ __device__ inline bool map_workgroup(int id, int H, int Hkv, int qb_begin, int qb_end, int* head, int* qb) {
+  const DispatchShape d = dispatch_shape(H, Hkv);
   const int x = id & 7, s = id >> 3;
   const int unit = (s / kUnit) * 8 + x, w = s % kUnit;
-  const int run = unit / Hkv;
-  const int kvh = (unit % Hkv + run) % Hkv;
-  const int from_end = run * unit_rows + w / group;
-  if (w >= group * unit_rows || from_end >= qb_end - qb_begin) return false;
+  const int run = unit / d.n_groups;
+  const int dg = (unit % d.n_groups + run) % d.n_groups;
+  const int from_end = run * d.unit_rows + w / d.set_heads;
+  const int in_group = (dg % d.sets) * d.set_heads + w % d.set_heads;   // head index inside its KV group
+  if (w >= d.set_heads * d.unit_rows || from_end >= qb_end - qb_begin || in_group >= d.group) return false;
   *qb = qb_end - 1 - from_end;
-  *head = kvh * group + w % group;
+  *head = (dg / d.sets) * d.group + in_group;
   return true;
 }
 
-// q-blocks per unit and grid size of a launch over [qb_begin, qb_end)
-inline int unit_rows_for(int H, int Hkv) {
-  const int group = H / Hkv;
-  return group >= kUnit ? 1 : kUnit / group;
-}
+// grid size of a launch over n_qblocks q-blocks
 inline int64_t grid_for(int H, int Hkv, int n_qblocks) {
-  const int ur = unit_rows_for(H, Hkv);
-  const int64_t runs = (n_qblocks + ur - 1) / ur;
-  return ((runs * Hkv + 7) / 8 * 8) * kUnit;
+  const DispatchShape d = dispatch_shape(H, Hkv);
+  const int64_t runs = (n_qblocks + d.unit_rows - 1) / d.unit_rows;
+  return ((runs * d.n_groups + 7) / 8 * 8) * kUnit;
 }
+
+// Token strides of K and V the tile copies can address (byte offsets inside a
+// 128-row tile are held in 32 bits), and a usable softmax scale.
+inline bool tile_stride_ok(int64_t sn) { return sn >= kHeadDim && sn <= ((int64_t)1 << 22); }
+inline bool scale_ok(float s) { return s > 0.f && s < 1e30f; }
 
 }  // namespace xattn

@@ -38,7 +38,6 @@ struct AttnParams {
   int idx_rows;             // q-block rows per head in col_idx / col_cnt (>= nqb)
   int H, Hkv, Lq, Lk, nqb, nkb;
   int qb_begin, qb_end;     // q-blocks handled by this launch
-  int unit_rows;            // q-blocks per dispatch unit
   int causal, kv_off;       // kv_off = Lk - Lq
   float scale_log2;         // softmax_scale * log2(e)
 };
@@ -55,7 +54,7 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   const int r = lane & 31, hh = lane >> 5;
 
   int head, qb;
-  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, p.unit_rows, p.qb_begin, p.qb_end, &head, &qb)) return;
+  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, p.qb_begin, p.qb_end, &head, &qb)) return;
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
@@ -305,6 +304,9 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   for (int64_t s : strides)
     if (s % 8) return XATTN_ERR_ALIGN;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return XATTN_ERR_ALIGN;
+  if (!tile_stride_ok(k_stride_n) || !tile_stride_ok(v_stride_n) || q_stride_n < kHeadDim || o_stride_n < kHeadDim)
+    return XATTN_ERR_SHAPE;
+  if (!scale_ok(softmax_scale)) return XATTN_ERR_SHAPE;
 
   AttnParams p;
   p.q = static_cast<const __bf16*>(q);
@@ -327,7 +329,6 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   if (q_block_begin < 0 || q_block_begin >= q_block_end || q_block_end > p.nqb) return XATTN_ERR_SHAPE;
   p.qb_begin = q_block_begin;
   p.qb_end = q_block_end;
-  p.unit_rows = unit_rows_for(p.H, p.Hkv);
   const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
   if (col_idx)

@@ -25,7 +25,6 @@ struct MassParams {
   float* mass;              // [H][nqb][nkb]
   int64_t q_sh, q_sn, k_sh, k_sn;
   int H, Hkv, Lq, Lk, nqb, nkb;
-  int unit_rows;
   int causal, kv_off;
   float scale_log2;
 };
@@ -38,7 +37,7 @@ __global__ __launch_bounds__(256, 2) void block_mass_kernel(MassParams p) {
   const int r = lane & 31, hh = lane >> 5;
 
   int head, qb;
-  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, p.unit_rows, 0, p.nqb, &head, &qb)) return;
+  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, 0, p.nqb, &head, &qb)) return;
   const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
@@ -250,6 +249,8 @@ extern "C" int xattn_block_mass(const void* q, const void* k, float* mass, int n
   for (int64_t s : strides)
     if (s % 8) return XATTN_ERR_ALIGN;
   if ((reinterpret_cast<uintptr_t>(q) & 15) || (reinterpret_cast<uintptr_t>(k) & 15)) return XATTN_ERR_ALIGN;
+  if (!tile_stride_ok(k_stride_n) || q_stride_n < kHeadDim) return XATTN_ERR_SHAPE;
+  if (!scale_ok(softmax_scale)) return XATTN_ERR_SHAPE;
   MassParams p;
   p.q = static_cast<const __bf16*>(q);
   p.k = static_cast<const __bf16*>(k);
@@ -258,7 +259,6 @@ extern "C" int xattn_block_mass(const void* q, const void* k, float* mass, int n
   p.H = num_heads; p.Hkv = num_kv_heads; p.Lq = q_len; p.Lk = k_len;
   p.nqb = (q_len + kBlk - 1) / kBlk;
   p.nkb = (k_len + kBlk - 1) / kBlk;
-  p.unit_rows = unit_rows_for(p.H, p.Hkv);
   p.causal = causal ? 1 : 0;
   p.kv_off = k_len - q_len;
   p.scale_log2 = softmax_scale * kLog2e;
