@@ -175,6 +175,29 @@ int xattn_decode_fwd(const void* q, const void* k, const void* v, void* out, voi
                      int64_t q_stride_h, int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h,
                      int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream);
 
+/* Allocation-free form of xattn_decode_fwd.  It has no counterpart in the
+ * reference: it exists for callers that cannot allocate device memory around
+ * the call - code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  Same arguments and result as xattn_decode_fwd minus the
+ * workspace: the per-range partial results live in a device array of
+ * XATTN_DECODE_STATIC_SCRATCH_BYTES that is part of the library (each GPU the
+ * library runs on holds its own copy until the process ends; its address on
+ * the current device is looked up on the first call there, so the device the
+ * stream belongs to must be current).  Problems whose
+ * xattn_decode_workspace_bytes() exceeds that size (more than 256 * 32
+ * (key range, query head) pairs: only with more than 256 KV heads) are refused
+ * with XATTN_ERR_WORKSPACE.  The function calls no hipMalloc / hipFree.  All
+ * calls on one GPU share the array: calls that may overlap on one GPU (two
+ * streams, two threads) race on it and must be ordered by the caller; nothing
+ * needs clearing between calls (every partial a launch reads it has written).
+ */
+#define XATTN_DECODE_STATIC_SCRATCH_BYTES (256 * 32 * 132 * 4)
+
+int xattn_decode_fwd_static(const void* q, const void* k, const void* v, void* out, int num_heads,
+                            int num_kv_heads, int k_len, int head_dim, int64_t q_stride_h,
+                            int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
+                            int64_t o_stride_h, float softmax_scale, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Stand-alone softmax + block sums over a score matrix in memory: the seam
  * softmax_fuse_block_sum, xattn/src/kernels.py:238-289 (kernels :5-156), for

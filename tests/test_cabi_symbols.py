@@ -70,6 +70,8 @@ def test_attention_entry_points_validate_strides_and_scale_before_launching():
     mass = lambda ksn, scale=0.1: lib.xattn_block_mass(a, a, a, 4, 2, 256, 256, 128, 128 * 256, 128, 128 * 256, ksn, 1,
                                                        scale, None)
     assert mass(big) == -4 and mass(64) == -4 and mass(128, scale=0.0) == -4
+    # the allocation-free decode form refuses what its built-in array cannot hold, before touching anything
+    assert lib.xattn_decode_fwd_static(a, a, a, a, 512 * 32, 512, 64, 128, 128, 8192, 128, 8192, 128, 128, 0.1, None) == -7
 
 
 def test_operator_refuses_cpu_tensors_and_wrong_dtypes():

@@ -18,6 +18,8 @@
 // four wavefronts combine (max, sum, unnormalised output) of their key ranges in
 // LDS and write one partial result per workgroup; a second small kernel merges
 // the workgroups of a head.
+#include <mutex>
+
 #include "xattn_common.h"
 #include "xattn_hip.h"
 
@@ -386,11 +388,14 @@ extern "C" size_t xattn_decode_workspace_bytes(int num_heads, int num_kv_heads, 
   return (size_t)(g.ranges_per_head / kDecWaves) * num_heads * kPartStride * sizeof(float);
 }
 
-extern "C" int xattn_decode_fwd(const void* q, const void* k, const void* v, void* out, void* workspace,
-                                size_t workspace_bytes, int num_heads, int num_kv_heads, int k_len, int head_dim,
-                                int64_t q_stride_h, int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h,
-                                int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream) {
-  if (!q || !k || !v || !out || !workspace) return XATTN_ERR_NULL;
+namespace {
+// Validates, fills the launch parameters and enqueues both kernels; `part` holds
+// part_bytes bytes of per-range partial results.
+int decode_launch(const void* q, const void* k, const void* v, void* out, void* part, size_t part_bytes,
+                  int num_heads, int num_kv_heads, int k_len, int head_dim, int64_t q_stride_h,
+                  int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
+                  int64_t o_stride_h, float softmax_scale, void* stream) {
+  if (!q || !k || !v || !out || !part) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
   if (num_heads / num_kv_heads > 32) return XATTN_ERR_HEADS;
@@ -399,11 +404,11 @@ extern "C" int xattn_decode_fwd(const void* q, const void* k, const void* v, voi
   for (int64_t s : strides)
     if (s % 8) return XATTN_ERR_ALIGN;
   auto a16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-  if (!a16(q) || !a16(k) || !a16(v) || !a16(workspace)) return XATTN_ERR_ALIGN;
+  if (!a16(q) || !a16(k) || !a16(v) || !a16(part)) return XATTN_ERR_ALIGN;
   // a tile's byte offsets are held in 32 bits
   if (k_stride_n > (1 << 22) || v_stride_n > (1 << 22) || k_stride_n < kHeadDim || v_stride_n < kHeadDim)
     return XATTN_ERR_SHAPE;
-  if (workspace_bytes < xattn_decode_workspace_bytes(num_heads, num_kv_heads, k_len)) return XATTN_ERR_WORKSPACE;
+  if (part_bytes < xattn_decode_workspace_bytes(num_heads, num_kv_heads, k_len)) return XATTN_ERR_WORKSPACE;
 
   const DecodeGeometry g = decode_geometry(num_kv_heads, k_len);
   DecodeParams p;
@@ -411,7 +416,7 @@ extern "C" int xattn_decode_fwd(const void* q, const void* k, const void* v, voi
   p.k = static_cast<const __bf16*>(k);
   p.v = static_cast<const __bf16*>(v);
   p.o = static_cast<__bf16*>(out);
-  p.part = static_cast<float*>(workspace);
+  p.part = static_cast<float*>(part);
   p.q_sh = q_stride_h; p.k_sh = k_stride_h; p.k_sn = k_stride_n;
   p.v_sh = v_stride_h; p.v_sn = v_stride_n; p.o_sh = o_stride_h;
   p.H = num_heads; p.Hkv = num_kv_heads; p.group = num_heads / num_kv_heads; p.Lk = k_len;
@@ -426,4 +431,63 @@ extern "C" int xattn_decode_fwd(const void* q, const void* k, const void* v, voi
   hipLaunchKernelGGL(decode_partial_kernel, dim3(grid), dim3(256), kDecLds, s, p);
   hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)num_heads), dim3(256), 0, s, p);
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
+}
+}  // namespace
+
+extern "C" int xattn_decode_fwd(const void* q, const void* k, const void* v, void* out, void* workspace,
+                                size_t workspace_bytes, int num_heads, int num_kv_heads, int k_len, int head_dim,
+                                int64_t q_stride_h, int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h,
+                                int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream) {
+  return decode_launch(q, k, v, out, workspace, workspace_bytes, num_heads, num_kv_heads, k_len, head_dim, q_stride_h,
+                       k_stride_h, k_stride_n, v_stride_h, v_stride_n, o_stride_h, softmax_scale, stream);
+}
+
+// ---------------------------------------------------------------------------
+// The same decode step for callers that may not allocate: the partial results
+// live in a device array that is part of this library's code object.  Every GPU
+// the library runs on holds its own copy of the array at its own address; the
+// address is looked up once per device and kept.  In host code the array's name
+// is only a handle for that lookup, never a pointer a kernel could use.
+namespace {
+// (256 / H_kv workgroups per KV head) x H query heads is at most 256 * 32
+// (range, head) pairs while H_kv <= 256 and H <= 32 H_kv.
+constexpr size_t kDecScratchBytes = (size_t)kDecCUs * 32 * kPartStride * sizeof(float);   // 4.125 MiB
+static_assert(kDecScratchBytes == XATTN_DECODE_STATIC_SCRATCH_BYTES, "header and kernel disagree on the scratch size");
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kDecScratchBytes];
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on first use).
+int scratch_of_current_device(void** ptr_out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return XATTN_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return XATTN_ERR_LAUNCH;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *ptr_out = g_scratch_ptr[dev];
+  return XATTN_OK;
+}
+}  // namespace
+
+extern "C" int xattn_decode_fwd_static(const void* q, const void* k, const void* v, void* out, int num_heads,
+                                       int num_kv_heads, int k_len, int head_dim, int64_t q_stride_h,
+                                       int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_h,
+                                       int64_t v_stride_n, int64_t o_stride_h, float softmax_scale, void* stream) {
+  const size_t need = xattn_decode_workspace_bytes(num_heads, num_kv_heads, k_len);
+  if (need == 0) {
+    if (num_heads <= 0 || num_kv_heads <= 0 || (num_kv_heads > 0 && num_heads % num_kv_heads)) return XATTN_ERR_HEADS;
+    return XATTN_ERR_SHAPE;
+  }
+  if (need > kDecScratchBytes) return XATTN_ERR_WORKSPACE;   // more (range, head) pairs than the array holds
+  void* ptr = nullptr;
+  const int rc = scratch_of_current_device(&ptr);
+  if (rc != XATTN_OK) return rc;
+  return decode_launch(q, k, v, out, ptr, kDecScratchBytes, num_heads, num_kv_heads, k_len, head_dim, q_stride_h,
+                       k_stride_h, k_stride_n, v_stride_h, v_stride_n, o_stride_h, softmax_scale, stream);
 }

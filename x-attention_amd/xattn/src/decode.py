@@ -15,7 +15,8 @@ from .Xattention import _stream_ptr
 __all__ = ["single_decode_with_kv_cache"]
 
 
-def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None, out=None, workspace=None):
+def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None, out=None, workspace=None,
+                                static_scratch=False):
     """``out[h] = softmax(q[h] . K[h // g]^T * sm_scale) V[h // g]``.
 
     q ``[H, 128]``; k, v ``[kv_len, H_kv, 128]`` for ``kv_layout="NHD"`` (the
@@ -25,7 +26,10 @@ def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None, out=Non
     taken as they are).  ``g = H / H_kv`` is at most 32.  ``sm_scale`` defaults
     to ``1/sqrt(128)``.  Returns ``[H, 128]`` in q's dtype.  ``workspace`` may
     carry a uint8 tensor of at least ``xattn_decode_workspace_bytes`` bytes to
-    avoid the per-call allocation.
+    avoid the per-call allocation.  ``static_scratch=True`` (with ``out`` given)
+    allocates nothing at all: the partial results go to a device array inside the
+    library, shared by every such call on the GPU - calls that may overlap on
+    one GPU must then be ordered by the caller.
     """
     lib = _hb.lib()
     if kv_layout not in ("NHD", "HND"):
@@ -62,7 +66,10 @@ def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None, out=Non
         sm_scale = 1.0 / math.sqrt(128)
     with torch.cuda.device(q.device):
         ws_bytes = lib.xattn_decode_workspace_bytes(heads, kv_heads, kv_len)
-        if workspace is None:
+        if static_scratch:
+            if workspace is not None:
+                raise ValueError("static_scratch and workspace exclude each other")
+        elif workspace is None:
             workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         elif workspace.numel() * workspace.element_size() < ws_bytes or workspace.device != q.device:
             raise ValueError(f"workspace must hold {ws_bytes} bytes on {q.device}")
@@ -70,6 +77,16 @@ def single_decode_with_kv_cache(q, k, v, kv_layout="NHD", sm_scale=None, out=Non
             out = torch.empty((heads, 128), dtype=q.dtype, device=q.device)
         elif out.shape != (heads, 128) or out.dtype != q.dtype or out.stride(1) != 1 or out.device != q.device:
             raise ValueError("out must be [H, 128], q's dtype and device, rows contiguous")
+        if static_scratch:
+            _hb.check(
+                lib.xattn_decode_fwd_static(
+                    q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), heads, kv_heads, kv_len, 128,
+                    q.stride(0), k.stride(0), k.stride(1), v.stride(0), v.stride(1), out.stride(0),
+                    float(sm_scale), _stream_ptr(q.device),
+                ),
+                "xattn_decode_fwd_static",
+            )
+            return out
         _hb.check(
             lib.xattn_decode_fwd(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), workspace.data_ptr(),

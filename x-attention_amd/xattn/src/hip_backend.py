@@ -35,6 +35,10 @@ _SIGNATURES = {
         c_i32,
         [c_vp] * 5 + [c_sz] + [c_i32] * 4 + [c_i64] * 6 + [c_f32, c_vp],
     ),
+    "xattn_decode_fwd_static": (
+        c_i32,
+        [c_vp] * 4 + [c_i32] * 4 + [c_i64] * 6 + [c_f32, c_vp],
+    ),
     "xattn_block_sparse_fwd": (
         c_i32,
         [c_vp] * 6 + [c_i64] + [c_i32] * 6 + [c_i64] * 8 + [c_i32, c_i32, c_i32, c_f32, c_vp],
