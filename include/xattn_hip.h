@@ -66,7 +66,9 @@ const char* xattn_error_string(int code);
  * reference's torch branch computes when k_len is a multiple of chunk_size,
  * Xattention.py:201).  causal == 0: every n is visible, zero-padded keys
  * included.  Rows m >= n_rq - (q_len_padded - q_len)/stride are all-zero
- * (Xattention.py:237-238).
+ * (Xattention.py:237-238; see zero_rows_from).  Zero-padded keys are never
+ * hidden: the reference's -inf over them (Xattention.py:201) is overwritten by
+ * the triangle of the only chunk whose rows reach them (:203-214).
  * Only query chunks [chunk_begin, chunk_end) are processed (rows of block_sums
  * outside them are left untouched), so a caller may pipeline chunks on streams.
  * `scores_out`, when non-null, receives the un-scaled scores of those chunks as
@@ -83,6 +85,17 @@ const char* xattn_error_string(int code);
  * input precision before the product, this sum is taken in fp32).
  * softmax == 0 writes block sums of exp(scaled score) over the visible keys
  * instead of softmax probabilities (Xattention.py:231-234).
+ * kdb > 1 subsamples the reshaped query rows (torch branch only,
+ * Xattention.py:88-93, 174-181, 217-222, 245): query row j takes the tokens of
+ * reshaped row j*kdb, sees (when causal) the keys of reshaped row j*kdb+kdb-1,
+ * and a query block sums block_size/stride/kdb rows; kdb must divide
+ * block_size/stride and needs the default reshape (num_slab_pairs == 0).
+ * zero_rows_from: query rows (after subsampling) at or beyond this index give
+ * all-zero block sums; negative = n_rq/kdb - (q_len_padded - q_len)/stride/kdb,
+ * the torch branch's padded tail.  The reference's Triton branch zeroes rows by
+ * their position on the key axis instead (xattn/src/kernels.py:70 with the
+ * real_q_len of Xattention.py:169): n_rq - (k_len_padded - k_len)/stride; padded
+ * query rows that rule leaves alone carry the uniform softmax of a zero query.
  * `workspace` must hold xattn_estimate_workspace_bytes(...) bytes, where
  * chunks_per_call is the largest chunk_end - chunk_begin used (<= 0: all chunks);
  * the function returns 0 for arguments the estimator rejects.
@@ -96,7 +109,7 @@ int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, v
                               int64_t q_stride_n, int64_t k_stride_h, int64_t k_stride_n, int stride,
                               int block_size, int chunk_size, int chunk_begin, int chunk_end, int causal,
                               int own_chunk_only, float scale, const int32_t* slab_pairs,
-                              int num_slab_pairs, int softmax, void* stream);
+                              int num_slab_pairs, int softmax, int kdb, int zero_rows_from, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Threshold block selection.  Replaces find_blocks_chunked,

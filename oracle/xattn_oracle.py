@@ -70,28 +70,32 @@ NEG_INF = float("-inf")
 # --------------------------------------------------------------------------- #
 # A3: antidiagonal (stride-S reversed reshape) scores
 # --------------------------------------------------------------------------- #
-def reshape_inverse(query_states, key_states, stride):
-    """Concatenation form of the stride-S reshape, select_mode="inverse", kdb=1.
+def reshape_inverse(query_states, key_states, stride, kdb=1):
+    """Concatenation form of the stride-S reshape, select_mode="inverse".
 
     Follows xattn/src/Xattention.py:84-94: keys take token ``n*S+i`` into
-    feature slab ``i``; queries take token ``m*S+(S-1-i)`` into slab ``i``.
+    feature slab ``i``; queries take token ``m*S*kdb+(S-1-i)`` into slab ``i``
+    (``kdb > 1`` keeps every kdb-th reshaped query row, the FIRST of each group).
     """
     rk = torch.cat([key_states[:, :, i::stride, :] for i in range(stride)], dim=-1)
     rq = torch.cat(
-        [query_states[:, :, (stride - 1 - i) :: stride, :] for i in range(stride)],
+        [query_states[:, :, (stride - 1 - i) :: (stride * kdb), :] for i in range(stride)],
         dim=-1,
     )
     return rq, rk
 
 
-def reshape_operands(query_states, key_states, stride, select_mode="inverse", perm=None):
+def reshape_operands(query_states, key_states, stride, select_mode="inverse", perm=None, kdb=1):
     """The reshaped (query, key) pair of every ``select_mode`` of the torch
-    branch, xattn/src/Xattention.py:72-135 (``kdb=1``).  ``perm`` stands for the
-    ``torch.randperm(stride)`` the reference draws for "random"."""
+    branch, xattn/src/Xattention.py:72-135.  ``perm`` stands for the
+    ``torch.randperm(stride)`` the reference draws for "random"; ``kdb`` enters
+    the "inverse" reshape only (:88-93)."""
     S, d = stride, query_states.shape[-1]
     rk = torch.cat([key_states[:, :, i::S, :] for i in range(S)], dim=-1)
     if select_mode in ("inverse", ""):
-        return reshape_inverse(query_states, key_states, stride)
+        return reshape_inverse(query_states, key_states, stride, kdb)
+    if kdb != 1:
+        raise ValueError("kdb != 1 only makes sense with select_mode='inverse'")
     if select_mode == "random":
         rq = torch.cat([query_states[:, :, int(perm[i]) :: S, :] for i in range(S)], dim=-1)
         return rq, rk
@@ -212,6 +216,8 @@ def estimate_chunk_block_sums(
     pad0_quirk,
     out_dtype,
     softmax=True,
+    kdb=1,
+    triton_rows=False,
 ):
     """Block sums of softmax(antidiagonal scores) for one query chunk.
 
@@ -221,15 +227,36 @@ def estimate_chunk_block_sums(
     keys of its own chunk.  ``pad0_quirk=False`` skips that line when there is
     no padding, which is what the reference's Triton branch computes
     (xattn/src/kernels.py:42-66 sweeps from key column 0).
+
+    ``kdb > 1`` (:174-181, :217-222, :245): the chunk holds ``rcs // kdb`` query
+    rows; the causal mask is built for ``rcs`` rows and every kdb-th row of it,
+    starting at ``kdb - 1``, is used - query row j (tokens of reshaped row
+    ``j*kdb``) sees keys up to reshaped position ``j*kdb + kdb - 1``; the rows
+    of the padded tail are the last ``q_reshaped_num_to_pad // kdb`` (a slice
+    ``-0:`` when that is 0, i.e. then the whole chunk); a query block sums
+    ``rbs // kdb`` rows.
+
+    ``triton_rows=True`` replaces the torch branch's padded-row rule by the
+    Triton branch's (xattn/src/kernels.py:70 with the ``real_q_len`` argument of
+    xattn/src/Xattention.py:169): a row is zeroed when its position on the key
+    axis is at or beyond the real (unpadded) reshaped key length, whatever the
+    query padding; padded query rows that rule leaves alone carry the uniform
+    softmax of an all-zero query.
     """
     bsz, heads = reshaped_query.shape[:2]
     rcs = chunk_size // stride
     rbs = block_size // stride
     offset_chunks = k_chunk_num - q_chunk_num
-    cq = reshaped_query[:, :, chunk_idx * rcs : (chunk_idx + 1) * rcs, :]
+    cq = reshaped_query[:, :, (chunk_idx * rcs) // kdb : (chunk_idx * rcs + rcs) // kdb, :]
     w = torch.matmul(cq, reshaped_key.transpose(2, 3))
     w = w / math.sqrt(head_dim) / stride / norm
     last_padded = chunk_idx == q_chunk_num - 1 and q_reshaped_num_to_pad != 0
+    if triton_rows:
+        assert kdb == 1
+        # key-axis position of this chunk's rows against the real reshaped key length
+        pos = (chunk_idx + offset_chunks) * rcs + torch.arange(rcs, device=w.device)
+        zero_rows = pos >= rcs * k_chunk_num - k_reshaped_num_to_pad
+        last_padded = False
     if causal:
         cm = torch.zeros((bsz, heads, rcs, rcs * k_chunk_num), device=w.device)
         if k_reshaped_num_to_pad > 0 or pad0_quirk:
@@ -240,16 +267,20 @@ def estimate_chunk_block_sums(
             torch.full((rcs, rcs), NEG_INF, device=w.device), diagonal=1
         )
         if last_padded:
-            cm[:, :, (-q_reshaped_num_to_pad):, :] = NEG_INF
+            cm[:, :, (-(q_reshaped_num_to_pad // kdb)):, :] = NEG_INF
         cm[..., c1:] = NEG_INF
+        cm = cm[:, :, kdb - 1 :: kdb, :]
         w = w + cm
     if softmax:
         w = F.softmax(w, dim=-1, dtype=torch.float32).to(out_dtype)
     else:
         w = torch.exp(w).to(out_dtype)   # Xattention.py:231-234
     if last_padded:
-        w[:, :, (-q_reshaped_num_to_pad):, :] = 0
-    sums = w.view(bsz, heads, rcs // rbs, rbs, -1, rbs).sum(dim=-1).sum(dim=-2)
+        w[:, :, (-(q_reshaped_num_to_pad // kdb)):, :] = 0
+    if triton_rows:
+        w = torch.nan_to_num(w, nan=0.0)
+        w[:, :, zero_rows, :] = 0
+    sums = w.view(bsz, heads, rcs // rbs, rbs // kdb, -1, rbs).sum(dim=-1).sum(dim=-2)
     return sums
 
 
@@ -273,14 +304,18 @@ def xattn_estimate(
 ):
     """(attn_sums, simple_masks), both ``[B, H, Nq_blocks_padded, Nk_blocks_padded]``.
 
-    Restates xattn/src/Xattention.py:13-299 for ``kdb=1`` on whatever device
-    the inputs live on (``perm``: the permutation "random" would draw).
-    ``use_triton`` is accepted for signature parity and ignored; the only
-    semantic difference between the two upstream branches that survives in
-    exact arithmetic is ``pad0_quirk`` (see :func:`estimate_chunk_block_sums`).
+    Restates xattn/src/Xattention.py:13-299 on whatever device the inputs live
+    on (``perm``: the permutation "random" would draw).  ``use_triton`` is
+    accepted for signature parity and ignored; which upstream branch is restated
+    is chosen by ``pad0_quirk``: ``True`` = the torch branch literally,
+    ``False`` = the Triton branch (keys of earlier chunks visible, and rows
+    zeroed by their key-axis position against the real key length; the two
+    row rules differ only when query and key padding differ).  ``kdb != 1``
+    exists in the torch branch only (the reference raises with ``use_triton``).
     """
-    if kdb != 1:
-        raise NotImplementedError("only kdb=1")
+    triton_rows = not pad0_quirk
+    if kdb != 1 and triton_rows:
+        raise ValueError("use_triton and kdb cannot be used together")
     bsz, kv_heads, k_len, head_dim = key_states.shape
     _, heads, q_len, _ = query_states.shape
     assert heads == kv_heads
@@ -294,7 +329,7 @@ def xattn_estimate(
     assert k_chunk_num >= q_chunk_num
     pk = F.pad(key_states, (0, 0, 0, k_pad), value=0) if k_pad else key_states
     pq = F.pad(query_states, (0, 0, 0, q_pad), value=0) if q_pad else query_states
-    rq, rk = reshape_operands(pq, pk, stride, select_mode, perm)
+    rq, rk = reshape_operands(pq, pk, stride, select_mode, perm, kdb)
     blocks_per_chunk = chunk_size // block_size
 
     sums, masks = [], []
@@ -316,6 +351,8 @@ def xattn_estimate(
             pad0_quirk=pad0_quirk,
             out_dtype=pq.dtype,
             softmax=softmax,
+            kdb=kdb,
+            triton_rows=triton_rows,
         )
         m = find_blocks_chunked(
             s,

@@ -182,3 +182,64 @@ def test_bad_slab_pairs_are_refused():
         estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, slab_pairs=[(8, 0)])      # offset outside the stride
     with pytest.raises(hb.XattnHipError):
         estimate_and_select(q.cuda(), k.cuda(), 8, 0.9, 512, slab_pairs=[(0, 0)] * 65)  # more than 64 pairs
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("kdb,S,C,L", [(2, 8, 512, 2048), (4, 8, 512, 1300), (2, 16, 1024, 3000), (4, 16, 2048, 4096),
+                                       (2, 4, 256, 1024), (4, 4, 256, 900), (2, 8, 256, 1016)])
+def test_kdb_matches_oracle(kdb, S, C, L, causal):
+    """Query-row subsampling of the reference's torch branch (xattn/src/Xattention.py:88-93,
+    174-181, 217-222, 245): block sums and mask against the oracle; (2, 8, 256, 1016) has
+    one padded reshaped row, fewer than kdb, which zeroes the whole last chunk (the slice [-0:])."""
+    from xattn.src.Xattention import estimate_and_select, xattn_estimate
+
+    q, k = _mk(4, 2, L, L, 40 + S + kdb, scale=1.5)
+    r = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=causal, use_triton=False, kdb=kdb)
+    want, want_mask = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, S, threshold=0.9,
+                                       chunk_size=C, causal=causal, kdb=kdb, pad0_quirk=True)
+    got = r["sums"].cpu()
+    assert got.shape == want[0].shape and torch.isfinite(got).all()
+    assert torch.allclose(got, want[0], rtol=2e-4, atol=2e-5), (got - want[0]).abs().max()
+    nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, causal, 0, C // 128)
+    assert outside == 0, (nbad, outside)
+    with pytest.raises(ValueError):
+        xattn_estimate(q.cuda(), k.cuda(), 128, S, chunk_size=C, kdb=kdb)          # use_triton=True, like the reference
+    _, m2 = xattn_estimate(q.cuda(), k.cuda(), 128, S, threshold=0.9, chunk_size=C, kdb=kdb, use_triton=False,
+                           causal=causal)
+    assert torch.equal(m2[0].cpu(), r["mask"].bool().cpu())
+
+
+@pytest.mark.parametrize("norm", [2, 0.5])
+@pytest.mark.parametrize("causal", [True, False])
+def test_norm_matches_oracle(norm, causal):
+    from xattn.src.Xattention import estimate_and_select
+
+    S, C, L = 8, 512, 1800
+    q, k = _mk(4, 2, L, L, 50, scale=1.5)
+    r = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=causal, norm=norm)
+    want, want_mask = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, S, threshold=0.9,
+                                       chunk_size=C, causal=causal, norm=norm, pad0_quirk=False)
+    assert torch.allclose(r["sums"].cpu(), want[0], rtol=2e-4, atol=2e-5)
+    nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, causal, 0, C // 128)
+    assert outside == 0, (nbad, outside)
+    plain = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=causal)["sums"]
+    assert not torch.allclose(plain, r["sums"], atol=1e-3)
+
+
+@pytest.mark.parametrize("use_triton", [True, False])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Lq,Lk,C", [(4000, 5000, 2048), (1000, 3000, 1024), (2100, 2300, 512)])
+def test_ragged_kv_longer_than_q_follows_each_branch_row_rule(Lq, Lk, C, causal, use_triton):
+    """Different query and key padding: the Triton branch zeroes rows by key-axis position against
+    the real key length (xattn/src/kernels.py:70), the torch branch the padded query tail."""
+    from xattn.src.Xattention import estimate_and_select
+
+    S = 8
+    q, k = _mk(4, 2, Lq, Lk, 60, scale=1.5)
+    r = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=causal, use_triton=use_triton)
+    want, want_mask = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, S, threshold=0.9,
+                                       chunk_size=C, causal=causal, pad0_quirk=not use_triton)
+    assert torch.allclose(r["sums"].cpu(), want[0], rtol=2e-4, atol=2e-5), (r["sums"].cpu() - want[0]).abs().max()
+    nq_p, nk_p = want_mask.shape[2], want_mask.shape[3]
+    nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, causal, nk_p - nq_p, C // 128)
+    assert outside == 0, (nbad, outside)

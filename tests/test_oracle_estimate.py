@@ -144,3 +144,109 @@ def test_default_chunk_rule():
     table = {1024: 2048, 2048: 2048, 4096: 4096, 16384: 16384, 32768: 8192, 65536: 4096, 131072: 2048, 119056: 2048, 1 << 20: 2048}
     for L, want in table.items():
         assert O.default_chunk_size(L) == want, L
+
+
+def loop_block_sums(q, k, S, bs, C, causal, *, kdb=1, norm=1.0, triton=False):
+    """Row-by-row restatement (python loops, fp64) of what the reference computes
+    per query chunk, written from the definitions rather than from tensor masks:
+
+    query row j of the padded, reshaped sequence stands for reshaped row ``j*kdb``
+    (tokens ``j*kdb*S + S-1-i``); when causal it sees reshaped keys up to position
+    ``j*kdb + kdb-1 + off`` (xattn/src/Xattention.py:204-222), zero-padded keys
+    included; the torch branch zeroes the last
+    ``q_pad_r // kdb`` rows of the last chunk (:237-238), the Triton branch the
+    rows whose key-axis position is at or beyond the real reshaped key length
+    (xattn/src/kernels.py:70, Xattention.py:169); a q-block sums ``rbs // kdb`` rows."""
+    d = q.shape[-1]
+    B, H, Lq, _ = q.shape
+    Lk = k.shape[2]
+    q_pad, k_pad = -Lq % C, -Lk % C
+    qp = torch.nn.functional.pad(q.double(), (0, 0, 0, q_pad))
+    kp = torch.nn.functional.pad(k.double(), (0, 0, 0, k_pad))
+    n_rq, n_rk = (Lq + q_pad) // S, (Lk + k_pad) // S
+    rbs, rcs = bs // S, C // S
+    off = n_rk - n_rq
+    rows = n_rq // kdb
+    rq_blk = rbs // kdb
+    out = torch.zeros(B, H, n_rq // rbs, n_rk // rbs, dtype=torch.float64)
+    q_pad_r, k_pad_r = q_pad // S, k_pad // S
+    last_chunk_first_row = (n_rq - rcs) // kdb
+    for h in range(H):
+        for j in range(rows):
+            m = j * kdb
+            s = torch.zeros(n_rk, dtype=torch.float64)
+            for i in range(S):
+                s += kp[0, h, i::S] @ qp[0, h, m * S + S - 1 - i]
+            s = s / math.sqrt(d) / S / norm
+            if causal:
+                vis = torch.arange(n_rk) <= m + kdb - 1 + off
+                # zero-padded keys are NOT hidden: the -inf the torch branch writes over them (:201) is
+                # overwritten by the triangle of the row's own chunk (:203-214), the only chunk whose rows
+                # reach them; they enter the softmax with logit 0 for every row at or beyond their position
+                if not triton and not k_pad_r:
+                    # the slice [..., -0:] of Xattention.py:201 hides every key before the row's own chunk
+                    vis &= torch.arange(n_rk) >= (m // rcs) * rcs + off
+                s = s.masked_fill(~vis, float("-inf"))
+            if triton:
+                zero = m + off >= n_rk - k_pad_r
+            else:
+                nz = q_pad_r // kdb
+                zero = q_pad_r != 0 and (j >= rows - nz if nz else j >= last_chunk_first_row)
+            if zero:
+                continue
+            p = torch.softmax(s, dim=0)
+            out[0, h, j // rq_blk] += p.view(n_rk // rbs, rbs).sum(-1)
+    return out
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("kdb,S,L", [(2, 8, 512), (4, 8, 512), (2, 4, 200), (4, 16, 1024), (2, 8, 456), (4, 8, 508)])
+def test_kdb_matches_row_loops(kdb, S, L, causal):
+    """Query-row subsampling of the torch branch (Xattention.py:76-83,174-181,217-222,245)."""
+    bs, C = 128, 256
+    q, k = make(L, H=1, seed=20 + kdb + S)
+    sums, mask = O.xattn_estimate(q, k, bs, S, threshold=0.9, chunk_size=C, causal=causal, kdb=kdb, pad0_quirk=True)
+    want = loop_block_sums(q, k, S, bs, C, causal, kdb=kdb)
+    assert sums.shape == want.shape
+    assert torch.allclose(sums.double(), want, atol=1e-5), (sums.double() - want).abs().max()
+    rbs = bs // S
+    full_rows = L // bs
+    if L % C == 0:
+        assert torch.allclose(sums.double().sum(-1)[..., :full_rows], torch.full((1, 1, full_rows), rbs / kdb, dtype=torch.float64), atol=1e-5)
+
+
+def test_kdb_is_refused_with_the_triton_branch():
+    q, k = make(256, H=1, seed=1)
+    with pytest.raises(ValueError):
+        O.xattn_estimate(q, k, 128, 8, chunk_size=256, kdb=2, pad0_quirk=False)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Lq,Lk,C", [(200, 456, 256), (300, 300, 256), (128, 600, 128), (250, 700, 256)])
+def test_triton_branch_zeroes_rows_by_key_position(Lq, Lk, C, causal):
+    """With k_len > q_len and different paddings the two branches zero different rows:
+    the Triton rule (kernels.py:70) against the row loops, the torch rule likewise."""
+    S, bs = 8, 32
+    q, k = make(Lq, H=1, seed=Lq + Lk, Lk=Lk)
+    for triton in (True, False):
+        sums, _ = O.xattn_estimate(q, k, bs, S, chunk_size=C, causal=causal, pad0_quirk=not triton)
+        want = loop_block_sums(q, k, S, bs, C, causal, triton=triton)
+        assert torch.allclose(sums.double(), want, atol=1e-5), (triton, (sums.double() - want).abs().max())
+    a, _ = O.xattn_estimate(q, k, bs, S, chunk_size=C, causal=causal, pad0_quirk=False)
+    b, _ = O.xattn_estimate(q, k, bs, S, chunk_size=C, causal=causal, pad0_quirk=True)
+    if (-Lq % C) != (-Lk % C):
+        assert not torch.allclose(a, b)           # the rules really differ on these shapes
+
+
+@pytest.mark.parametrize("norm", [2, 0.5])
+def test_norm_divides_the_logits(norm):
+    S, bs, L = 8, 32, 256
+    q, k = make(L, H=1, seed=31)
+    sums, _ = O.xattn_estimate(q, k, bs, S, chunk_size=128, causal=True, norm=norm, pad0_quirk=False)
+    want = loop_block_sums(q, k, S, bs, 128, True, norm=norm, triton=True)
+    assert torch.allclose(sums.double(), want, atol=1e-5)
+    # equivalent to scaling the queries
+    other, _ = O.xattn_estimate(q / norm, k, bs, S, chunk_size=128, causal=True, pad0_quirk=False)
+    assert torch.allclose(sums, other, atol=1e-6)
+    plain, _ = O.xattn_estimate(q, k, bs, S, chunk_size=128, causal=True, pad0_quirk=False)
+    assert not torch.allclose(sums, plain, atol=1e-3)

@@ -41,11 +41,13 @@ struct EstParams {
   float* sums;     // [H][nqb][nkb] output block sums
   int H, Hkv, Lq, Lk, S, rbs;
   int n_rq, n_rk, nkb, nqb, nT;
-  int rcs;                  // reshaped rows per chunk
-  int row_begin, row_end;   // reshaped query rows handled by this call
+  int rcs;                  // reshaped keys per chunk
+  int kdb;                  // query-row subsampling: query row m stands for reshaped row m * kdb
+  int rcs_q, rbs_q;         // query rows per chunk / per query block (rcs / kdb, rbs / kdb)
+  int row_begin, row_end;   // query rows handled by this call
   int rows;                 // row_end - row_begin (pitch of P / Mt / Lt)
-  int off;                  // n_rk - n_rq: position of query row 0 on the key axis
-  int real_rows;            // query rows >= real_rows are padding
+  int off;                  // position of reshaped row 0 on the key axis: n_rk - n_rq * kdb
+  int real_rows;            // query rows >= real_rows give all-zero block sums
   int causal, own_chunk_only;
   int no_softmax;           // block sums of exp(scaled score) instead of softmax probabilities
   float scale_log2;
@@ -60,11 +62,13 @@ struct EstParams {
 };
 
 // first / last visible reshaped key of reshaped query row m
-__device__ __forceinline__ int row_lo(const EstParams& p, int m) {
-  return (p.causal && p.own_chunk_only) ? (m / p.rcs) * p.rcs + p.off : 0;
+// (with kdb > 1 the row's causal limit is that of the LAST reshaped row of its
+// group, xattn/src/Xattention.py:217-222, while its tokens are those of the first, :88-93)
+__host__ __device__ inline int row_lo(const EstParams& p, int m) {
+  return (p.causal && p.own_chunk_only) ? (m / p.rcs_q) * p.rcs + p.off : 0;
 }
-__device__ __forceinline__ int row_hi(const EstParams& p, int m) {
-  return p.causal ? m + p.off : p.n_rk - 1;
+__host__ __device__ inline int row_hi(const EstParams& p, int m) {
+  return p.causal ? m * p.kdb + p.kdb - 1 + p.off : p.n_rk - 1;
 }
 
 // A k-step slab is 256 rows x 64 bf16 (one 128-byte line per row) per operand,
@@ -160,10 +164,10 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   // sequence end (or the tile's end), so lane offsets stay small whatever the
   // token stride, and tokens past the real length read as zeros.
   const int64_t q_snb = p.q_sn * 2, k_snb = p.k_sn * 2;
-  const int64_t q_tok0 = (int64_t)m0 * p.S, k_tok0 = (int64_t)n0 * p.S;
+  const int64_t q_tok0 = (int64_t)m0 * p.S * p.kdb, k_tok0 = (int64_t)n0 * p.S;
   const int64_t q_left = p.Lq - q_tok0, k_left = p.Lk - k_tok0;
   const int64_t span = (int64_t)kTile * p.S;
-  const int64_t q_rows = q_left < 0 ? 0 : (q_left < span ? q_left : span);
+  const int64_t q_rows = q_left < 0 ? 0 : (q_left < span * p.kdb ? q_left : span * p.kdb);
   const int64_t k_rows = k_left < 0 ? 0 : (k_left < span ? k_left : span);
   const __amdgpu_buffer_rsrc_t qres = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(qbase + (q_rows > 0 ? q_tok0 * p.q_sn : 0)), 0, (int)(q_rows * q_snb), 0x00020000);
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   const int steps = (kTable ? p.n_pairs : p.S) * 2;
   int voffK[4], voffQ[4];
   slab_offsets(k_snb, p.S, lane, wave, voffK);
-  slab_offsets(q_snb, p.S, lane, wave, voffQ);
+  slab_offsets(q_snb, p.S * p.kdb, lane, wave, voffQ);
   auto step_off_k = [&](int t) {
     const int i = kTable ? (p.pairs[t >> 1] & 15) : (t >> 1);
     return i * (int)k_snb + (t & 1) * kDepth * 2;
@@ -443,6 +447,68 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
   }
 }
 
+// The same normalisation for subsampled query rows (kdb > 1): a query block then
+// has rbs / kdb rows (possibly fewer than four), which the vectorised kernel
+// above does not handle.  One workgroup per (query block, head): thread
+// (row = tid % 32, part = tid / 32) folds every 8th key tile into the row's
+// statistics, then each thread owns key blocks tid, tid + 256, ...
+__global__ __launch_bounds__(256) void estimate_normalize_rows_kernel(EstParams p) {
+  __shared__ float redM[8][32];
+  __shared__ float redL[8][32];
+  __shared__ float rowM[32];
+  __shared__ float rowInv[32];
+  const int tid = threadIdx.x, row = tid & 31, part = tid >> 5;
+  const int head = blockIdx.y;
+  const int m0 = p.row_begin + blockIdx.x * p.rbs_q;     // first query row of the block
+  const float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
+  const float* Mst = p.Mt + (int64_t)head * p.nT * p.rows;
+  const float* Lst = p.Lt + (int64_t)head * p.nT * p.rows;
+  const bool row_ok = row < p.rbs_q && m0 + row < p.row_end;
+  const int m = row_ok ? m0 + row : m0;
+  const int mrel = m - p.row_begin;
+  const int lo = row_lo(p, m);
+  int hi = row_hi(p, m);
+  hi = hi < p.n_rk - 1 ? hi : p.n_rk - 1;
+  float M = -INFINITY, L = 0.f;
+  for (int T = lo / kSub + part; T <= hi / kSub; T += 8) {
+    const float mt = Mst[(int64_t)T * p.rows + mrel];
+    const float lt = Lst[(int64_t)T * p.rows + mrel];
+    const float Mn = fmaxf(M, mt);
+    const float safe = (Mn == -INFINITY) ? 0.f : Mn;
+    L = L * fast_exp2(M - safe) + lt * fast_exp2(mt - safe);
+    M = Mn;
+  }
+  redM[part][row] = M;
+  redL[part][row] = L;
+  __syncthreads();
+  if (part == 0) {
+    float Mr = -INFINITY;
+    for (int w = 0; w < 8; ++w) Mr = fmaxf(Mr, redM[w][row]);
+    const float safe = (Mr == -INFINITY) ? 0.f : Mr;
+    float Lr = 0.f;
+    for (int w = 0; w < 8; ++w) Lr += redL[w][row] * fast_exp2(redM[w][row] - safe);
+    const bool real = row_ok && m < p.real_rows && Lr > 0.f;
+    rowM[row] = p.no_softmax ? 0.f : safe;
+    rowInv[row] = real ? (p.no_softmax ? 1.f : 1.f / Lr) : 0.f;
+  }
+  __syncthreads();
+  float* out = p.sums + ((int64_t)head * p.nqb + m0 / p.rbs_q) * p.nkb;
+  for (int kb = tid; kb < p.nkb; kb += 256) {
+    const int T = (kb * p.rbs) / kSub;
+    float acc = 0.f;
+    for (int r = 0; r < p.rbs_q; ++r) {
+      const int mr = m0 + r;
+      if (mr >= p.row_end || rowInv[r] == 0.f) continue;
+      int h2 = row_hi(p, mr);
+      h2 = h2 < p.n_rk - 1 ? h2 : p.n_rk - 1;
+      if (kb < row_lo(p, mr) / p.rbs || kb > h2 / p.rbs) continue;
+      const int rel = mr - p.row_begin;
+      acc += Pst[(int64_t)kb * p.rows + rel] * fast_exp2(Mst[(int64_t)T * p.rows + rel] - rowM[r]) * rowInv[r];
+    }
+    out[kb] = acc;
+  }
+}
+
 }  // namespace xattn
 
 using namespace xattn;
@@ -460,7 +526,7 @@ hipError_t launch_gemm(const EstParams& p, dim3 grid, size_t lds, hipStream_t s)
 }
 
 struct Geometry {
-  int q_pad, k_pad, n_rq, n_rk, nqb, nkb, nT, rcs, q_chunks;
+  int q_pad, k_pad, n_rq, n_rk, nqb, nkb, nT, rcs, q_chunks;   // n_rq: reshaped query rows before subsampling
 };
 
 bool geometry(int q_len, int k_len, int stride, int block_size, int chunk_size, Geometry* g) {
@@ -492,7 +558,7 @@ extern "C" size_t xattn_estimate_workspace_bytes(int num_heads, int q_len, int k
   if (num_heads <= 0 || block_size != 128 || (stride != 4 && stride != 8 && stride != 16)) return 0;
   if (!geometry(q_len, k_len, stride, block_size, chunk_size, &g)) return 0;
   int c = (chunks_per_call <= 0 || chunks_per_call > g.q_chunks) ? g.q_chunks : chunks_per_call;
-  return workspace_bytes(num_heads, g, c * g.rcs);
+  return workspace_bytes(num_heads, g, c * g.rcs);   // (an upper bound when query rows are subsampled)
 }
 
 extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, void* workspace,
@@ -502,7 +568,7 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
                                          int64_t k_stride_n, int stride, int block_size, int chunk_size,
                                          int chunk_begin, int chunk_end, int causal, int own_chunk_only,
                                          float scale, const int32_t* slab_pairs, int num_slab_pairs,
-                                         int softmax, void* stream) {
+                                         int softmax, int kdb, int zero_rows_from, void* stream) {
   if (!q || !k || !block_sums || !workspace) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
@@ -510,6 +576,10 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   Geometry g;
   if (!geometry(q_len, k_len, stride, block_size, chunk_size, &g)) return XATTN_ERR_SHAPE;
   if (chunk_begin < 0 || chunk_end > g.q_chunks || chunk_begin >= chunk_end) return XATTN_ERR_SHAPE;
+  // query-row subsampling must divide the rows of a chunk and of a query block; only the
+  // antidiagonal reshape has it (xattn/src/Xattention.py:88-93)
+  if (kdb < 1 || (block_size / stride) % kdb || g.rcs % kdb || (kdb > 1 && num_slab_pairs != 0)) return XATTN_ERR_SHAPE;
+  if (!(scale > 0.f) || !(scale < 1e30f)) return XATTN_ERR_SHAPE;
   if (q_stride_h % 8 || q_stride_n % 8 || k_stride_h % 8 || k_stride_n % 8) return XATTN_ERR_ALIGN;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k)) & 15) return XATTN_ERR_ALIGN;
 
@@ -519,17 +589,19 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.q_sh = q_stride_h; p.q_sn = q_stride_n; p.k_sh = k_stride_h; p.k_sn = k_stride_n;
   if (q_stride_n < kHeadDim || k_stride_n < kHeadDim) return XATTN_ERR_ALIGN;
   // one 256-row tile (256 * stride tokens) must span less than 2^31 bytes
-  if ((int64_t)(kTile + 1) * stride * q_stride_n * 2 >= 0x7fffffff ||
+  if ((int64_t)(kTile + 1) * stride * kdb * q_stride_n * 2 >= 0x7fffffff ||
       (int64_t)(kTile + 1) * stride * k_stride_n * 2 >= 0x7fffffff)
     return XATTN_ERR_SHAPE;
   p.H = num_heads; p.Hkv = num_kv_heads; p.Lq = q_len; p.Lk = k_len; p.S = stride;
   p.rbs = block_size / stride;
-  p.n_rq = g.n_rq; p.n_rk = g.n_rk; p.nkb = g.nkb; p.nqb = g.nqb; p.nT = g.nT; p.rcs = g.rcs;
-  p.row_begin = chunk_begin * g.rcs;
-  p.row_end = chunk_end * g.rcs;
+  p.n_rq = g.n_rq / kdb; p.n_rk = g.n_rk; p.nkb = g.nkb; p.nqb = g.nqb; p.nT = g.nT; p.rcs = g.rcs;
+  p.kdb = kdb; p.rcs_q = g.rcs / kdb; p.rbs_q = p.rbs / kdb;
+  p.row_begin = chunk_begin * p.rcs_q;
+  p.row_end = chunk_end * p.rcs_q;
   p.rows = p.row_end - p.row_begin;
   p.off = g.n_rk - g.n_rq;
-  p.real_rows = g.n_rq - g.q_pad / stride;
+  // default: the torch branch's rule for kdb = 1 (the padded tail, xattn/src/Xattention.py:237-238)
+  p.real_rows = zero_rows_from >= 0 ? zero_rows_from : p.n_rq - g.q_pad / stride / kdb;
   p.causal = causal ? 1 : 0;
   p.own_chunk_only = own_chunk_only ? 1 : 0;
   p.scale_log2 = scale * kLog2e;
@@ -557,9 +629,9 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   for (int r = 0; r < p.nMT; ++r) {   // same visibility rule as the kernel's row_lo / row_hi
     const int mfirst = p.row_begin + r * kTile;
     const int mlast = (mfirst + kTile - 1 < p.row_end ? mfirst + kTile - 1 : p.row_end - 1);
-    int hi = (p.causal ? mlast + p.off : p.n_rk - 1) / kTile;
+    int hi = row_hi(p, mlast) / kTile;
     hi = hi < p.nNT - 1 ? hi : p.nNT - 1;
-    const int lo = ((p.causal && p.own_chunk_only) ? (mfirst / p.rcs) * p.rcs + p.off : 0) / kTile;
+    const int lo = row_lo(p, mfirst) / kTile;
     p.tiles_per_head += hi - lo + 1;
   }
   p.total_tiles = (int64_t)p.tiles_per_head * num_heads;
@@ -573,19 +645,21 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   switch (p.rbs) {
     case 8:
       e = launch_gemm<8>(p, grid1, lds, s);
-      if (e != hipSuccess) return XATTN_ERR_LAUNCH;
-      hipLaunchKernelGGL(estimate_normalize_kernel<8>, grid2, dim3(256), 0, s, p);
+      if (e == hipSuccess && kdb == 1) hipLaunchKernelGGL(estimate_normalize_kernel<8>, grid2, dim3(256), 0, s, p);
       break;
     case 16:
       e = launch_gemm<16>(p, grid1, lds, s);
-      if (e != hipSuccess) return XATTN_ERR_LAUNCH;
-      hipLaunchKernelGGL(estimate_normalize_kernel<16>, grid2, dim3(256), 0, s, p);
+      if (e == hipSuccess && kdb == 1) hipLaunchKernelGGL(estimate_normalize_kernel<16>, grid2, dim3(256), 0, s, p);
       break;
     default:
       e = launch_gemm<32>(p, grid1, lds, s);
-      if (e != hipSuccess) return XATTN_ERR_LAUNCH;
-      hipLaunchKernelGGL(estimate_normalize_kernel<32>, grid2, dim3(256), 0, s, p);
+      if (e == hipSuccess && kdb == 1) hipLaunchKernelGGL(estimate_normalize_kernel<32>, grid2, dim3(256), 0, s, p);
       break;
+  }
+  if (e != hipSuccess) return XATTN_ERR_LAUNCH;
+  if (kdb != 1) {
+    const dim3 grid3(p.rows / p.rbs_q, num_heads);
+    hipLaunchKernelGGL(estimate_normalize_rows_kernel, grid3, dim3(256), 0, s, p);
   }
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
 }

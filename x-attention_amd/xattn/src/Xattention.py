@@ -101,8 +101,9 @@ class _Plan:
     """Geometry, buffers and kernel launchers of one estimate -> select pass."""
 
     def __init__(self, query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs=None, softmax=True):
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs=None, softmax=True, kdb=1):
         self.lib = _hb.lib()
+        self.kdb = int(kdb)
         self.softmax = bool(softmax)
         self.n_pairs = 0 if slab_pairs is None else len(slab_pairs)
         self.pairs = None
@@ -124,6 +125,13 @@ class _Plan:
             raise AssertionError("query heads must be a multiple of key/value heads")
         if chunk_size % block_size:
             raise AssertionError("chunk_size must be a multiple of block_size")
+        if self.kdb != 1:
+            if use_triton:
+                raise ValueError("use_triton and kdb cannot be used together")     # xattn/src/Xattention.py:140-141
+            if self.kdb < 1 or (block_size // stride) % self.kdb or self.n_pairs:
+                raise ValueError("kdb must divide block_size // stride and needs select_mode='inverse'")
+        if not norm > 0:
+            raise ValueError("norm must be positive")
         self.stride, self.chunk_size, self.block_size = stride, chunk_size, block_size
         self.causal, self.keep_sink, self.keep_recent = bool(causal), bool(keep_sink), bool(keep_recent)
         dev = self.dev = q.device
@@ -135,6 +143,19 @@ class _Plan:
         self.blocks_per_chunk = chunk_size // block_size
         self.own_chunk_only = self.causal and (not use_triton) and k_pad == 0
         self.scale = 1.0 / math.sqrt(128) / stride / norm
+        # Query rows (after subsampling) from which the block sums are all-zero.  Torch branch: the last
+        # q_pad // stride // kdb rows of the last chunk - all of that chunk when that count is 0 but there is
+        # padding, the slice [-0:] of xattn/src/Xattention.py:237-238.  Triton branch: rows whose position on
+        # the key axis is at or beyond the real reshaped key length (xattn/src/kernels.py:70, Xattention.py:169).
+        n_rq = (self.q_len + q_pad) // stride // self.kdb
+        if use_triton:
+            self.zero_rows_from = max(0, n_rq - k_pad // stride)
+        elif q_pad // stride == 0:
+            self.zero_rows_from = n_rq
+        elif q_pad // stride // self.kdb == 0:
+            self.zero_rows_from = n_rq - chunk_size // stride // self.kdb
+        else:
+            self.zero_rows_from = n_rq - q_pad // stride // self.kdb
         self.list_cols = (self.k_len + block_size - 1) // block_size
         # The estimator's workspace grows with (query rows per call) x (key blocks); very long
         # sequences are processed in groups of query chunks that keep it under WORKSPACE_LIMIT.
@@ -151,7 +172,7 @@ class _Plan:
             self.scores = None
             if dump_scores:
                 self.scores = torch.zeros(
-                    (self.heads, (self.q_len + q_pad) // stride, (self.k_len + k_pad) // stride),
+                    (self.heads, (self.q_len + q_pad) // stride // self.kdb, (self.k_len + k_pad) // stride),
                     dtype=torch.float32, device=dev)
             self.tau = _tau_per_head(threshold, self.heads, dev)
             self.mask = torch.empty((self.heads, self.nqb, self.nkb), dtype=torch.uint8, device=dev)
@@ -174,7 +195,7 @@ class _Plan:
                 q.stride(1), q.stride(2), k.stride(1), k.stride(2),
                 self.stride, self.block_size, self.chunk_size, chunk_begin, chunk_end,
                 int(self.causal), int(self.own_chunk_only), self.scale, self.pairs, self.n_pairs,
-                int(self.softmax), stream,
+                int(self.softmax), self.kdb, self.zero_rows_from, stream,
             ),
             "xattn_estimate_block_sums",
         )
@@ -214,6 +235,7 @@ def estimate_and_select(
     marks=None,
     slab_pairs=None,
     softmax=True,
+    kdb=1,
 ):
     """Runs the estimator and selection kernels over all query chunks, one launch each.
 
@@ -226,7 +248,7 @@ def estimate_and_select(
     and after selection (for per-kernel timing).
     """
     plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs, softmax)
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs, softmax, kdb)
     with torch.cuda.device(plan.dev):
         stream = _stream_ptr(plan.dev)
         _mark(marks, "estimate_begin")
@@ -262,14 +284,17 @@ def xattn_estimate(
     "double", "triple"; the reference has the last four in its torch branch only,
     Xattention.py:72-135) and ``softmax=False`` (:231-234) run on the same
     kernel; "random" draws ``torch.randperm(stride)`` like the reference.
-    ``kdb != 1`` (query rows subsampled, no caller uses it) is not provided.
+    ``kdb != 1`` (every kdb-th reshaped query row, :88-93, :174-181, :217-222,
+    :245) exists in the reference's torch branch only: it needs
+    ``use_triton=False`` (the reference raises otherwise, :140-141) and the
+    default ``select_mode``.
     """
-    if kdb != 1:
-        raise ValueError("kdb != 1 is not supported by the fused estimator")
+    if kdb != 1 and use_triton:
+        raise ValueError("use_triton and kdb cannot be used together")
     r = estimate_and_select(
         query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
         use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
-        want_lists=False, slab_pairs=slab_pairs_for(select_mode, stride), softmax=softmax,
+        want_lists=False, slab_pairs=slab_pairs_for(select_mode, stride), softmax=softmax, kdb=kdb,
     )
     attn_sums = r["sums"].to(query_states.dtype).unsqueeze(0)
     simple_masks = r["mask"].view(torch.bool).unsqueeze(0)
@@ -352,17 +377,15 @@ def Xattention_prefill(
     batch_size, _, k_len, _ = key_states.shape
     assert block_size == 128
     assert batch_size == 1
-    if kdb != 1:
-        raise ValueError("kdb != 1 is not supported by the fused estimator")
     if chunk_size is None:
         chunk_size = default_chunk_size(k_len)
     if pipeline_chunks:
         return _prefill_pipelined(query_states, key_states, value_states, stride, norm, threshold, block_size,
-                                  use_triton, causal, chunk_size, keep_sink, keep_recent)
+                                  use_triton, causal, chunk_size, keep_sink, keep_recent, kdb)
     r = estimate_and_select(
         query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
         use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
-        want_lists=True,
+        want_lists=True, kdb=kdb,
     )
     return block_sparse_attention(
         query_states, key_states, value_states, r["col_idx"], r["col_cnt"], causal=causal
@@ -381,7 +404,7 @@ def _streams(dev):
 
 
 def _prefill_pipelined(query_states, key_states, value_states, stride, norm, threshold, block_size, use_triton,
-                       causal, chunk_size, keep_sink, keep_recent):
+                       causal, chunk_size, keep_sink, keep_recent, kdb=1):
     """Chunk-by-chunk orchestration on three HIP streams: the estimator of query
     chunk c runs on the caller's stream, the selection of chunk c on a second
     stream as soon as its block sums exist, and the attention of chunk c's query
@@ -390,7 +413,7 @@ def _prefill_pipelined(query_states, key_states, value_states, stride, norm, thr
     leaves idle.  The caller's stream waits for both side streams before the
     function returns, which also makes every temporary safe to free."""
     plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, True, False)
+                 keep_sink, keep_recent, block_size, True, False, kdb=kdb)
     dev = plan.dev
     q = plan.q
     k = plan.k

@@ -19,7 +19,7 @@ _SIGNATURES = {
     "xattn_estimate_block_sums": (
         c_i32,
         [c_vp, c_vp, c_vp, c_vp, c_sz, c_vp] + [c_i32] * 5 + [c_i64] * 4 + [c_i32] * 7
-        + [c_f32, ctypes.POINTER(c_i32), c_i32, c_i32, c_vp],
+        + [c_f32, ctypes.POINTER(c_i32), c_i32, c_i32, c_i32, c_i32, c_vp],
     ),
     "xattn_select_blocks": (
         c_i32,
