@@ -11,16 +11,22 @@ from . import xattn_oracle as O
 TAU_BAND = 1e-5      # masks may differ only on blocks whose cumulative mass is this close to tau
 
 
-def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None):
+def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None):
     """Compares two block masks given the block sums both were selected from.
 
-    Returns (n_mismatch, n_outside_band).  A mismatching block is inside the band
-    when the mass the selection rule compares against tau * total for it (or for
-    a block of equal sum) is within TAU_BAND * total of tau * total - the only
-    place where summation order or tie order can flip a decision.  Column 0 is
-    also set whenever any rank is left out, so it may flip with whichever block
-    sits at the crossing.  Forced blocks and blocks beyond the diagonal are
-    never inside the band.
+    Returns a dict: ``mismatches``; ``in_band`` - mismatching blocks for which the
+    mass the selection rule compares against tau * total (for it or for a block of
+    equal sum) is within TAU_BAND * total of tau * total, the only place where
+    summation order can flip a decision (column 0 is also set whenever any rank is
+    left out, so it may flip with whichever block sits at the crossing);
+    ``ties`` - mismatching blocks that belong to a run of equal sums (equal to
+    within TAU_BAND * total, the same tolerance) which the threshold crossing cuts
+    through, with both masks keeping as many of them as the rule allows: which members of
+    such a run are kept is the order an unstable sort happens to give (the
+    reference uses torch.sort, xattn/src/utils.py:110,126,150) or, for sums that
+    differ in the last bits, the order rounding gives;
+    ``outside`` - everything else, i.e. real disagreements.  Forced blocks and
+    blocks beyond the diagonal are never excused.
     """
     import numpy as np
 
@@ -33,7 +39,7 @@ def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_c
     if taus.numel() == 1:
         taus = taus.expand(H)
     bad = (got != want).nonzero().tolist()
-    outside = 0
+    outside = ties = 0
     rows = {}
     for h, i, j in bad:
         diag = i + diag_offset
@@ -49,19 +55,41 @@ def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_c
             cols = np.array([c for c in range(limit) if c not in forced], dtype=np.int64)
             vals = row[cols]
             order = np.lexsort((cols, -vals))          # descending sum, ascending column among equals
-            vals = vals[order]
+            vals, cols = vals[order], cols[order]
             base = float(sum(row[c] for c in forced if c < nk))
             before = base + np.concatenate(([0.0], np.cumsum(vals)[:-1])) if len(vals) else np.zeros(0)
             if one_forced and len(vals):
                 before = before - np.concatenate(([0.0], vals[:-1]))
                 before[0] = 0.0
-            near = np.abs(before - taus[h].item() * total) <= TAU_BAND * max(total, 1e-30)
-            rows[(h, i)] = (row, vals, near)
-        row, vals, near = rows[(h, i)]
-        ok = bool((near & (vals == row[j])).any()) or (j == 0 and bool(near.any()))
-        if not ok:
-            outside += 1
-    return len(bad), outside
+            need = taus[h].item() * total
+            near = np.abs(before - need) <= TAU_BAND * max(total, 1e-30)
+            rows[(h, i)] = (row, vals, cols, near, before < need)
+        row, vals, cols, near, keep = rows[(h, i)]
+        same = np.abs(vals - row[j]) <= TAU_BAND * max(float(row.sum()), 1e-30)
+        if bool((near & same).any()) or (j == 0 and bool(near.any())):
+            continue
+        run = cols[same]
+        kept = int(keep[same].sum())
+        cut = 0 < kept < len(run)
+        if cut:
+            # any `kept` members of the run may be the chosen ones; column 0, when it is a member, is set
+            # anyway (unselected ranks scatter to it), so a mask may show one chosen member fewer beside it
+            rest = run[run != 0]
+            free0 = len(rest) != len(run)
+            counts = {kept - 1, kept} if free0 else {kept}
+            ok = all(int(m[h, i][rest].sum()) in counts and (not free0 or bool(m[h, i][0])) for m in (got, want))
+            if ok:
+                ties += 1
+                continue
+        outside += 1
+    return {"mismatches": len(bad), "in_band": len(bad) - outside - ties, "ties": ties, "outside": outside}
+
+
+def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None):
+    """(number of mismatching blocks, number of them that the parity contract does
+    not excuse) - see :func:`mask_mismatch_detail`."""
+    d = mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_chunk)
+    return d["mismatches"], d["outside"]
 
 
 def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal, pad0_quirk, sums_got=None):
@@ -70,7 +98,7 @@ def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal
     compares its block mask with ``got_mask`` (that head's ``[Nq_p, Nk_p]`` mask
     from the path under test).
 
-    Returns a dict: blocks, mismatches, in_band (mismatches the contract
+    Returns a dict: blocks, mismatches, in_band and ties (mismatches the contract
     allows), outside_band, density of the oracle's mask over the padded grid
     and, when ``sums_got`` is given, the largest absolute difference of the
     block sums.
@@ -87,9 +115,9 @@ def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal
                                             causal=causal, pad0_quirk=pad0_quirk)
     nq_p, nk_p = want_mask.shape[2], want_mask.shape[3]
     got = got_mask.reshape(1, nq_p, nk_p)
-    nbad, outside = mask_mismatch_report(want_sums[0], got, want_mask[0], tau, causal, nk_p - nq_p, chunk_size // 128)
-    rep = {"head": int(head), "blocks": int(want_mask.numel()), "mismatches": int(nbad), "in_band": int(nbad - outside),
-           "outside_band": int(outside), "oracle_density": round(float(want_mask.float().mean()), 5)}
+    d = mask_mismatch_detail(want_sums[0], got, want_mask[0], tau, causal, nk_p - nq_p, chunk_size // 128)
+    rep = {"head": int(head), "blocks": int(want_mask.numel()), "mismatches": d["mismatches"], "in_band": d["in_band"],
+           "ties": d["ties"], "outside_band": d["outside"], "oracle_density": round(float(want_mask.float().mean()), 5)}
     if sums_got is not None:
         rep["sums_max_abs_diff"] = float((sums_got.detach().float().cpu().reshape(nq_p, nk_p) - want_sums[0, 0]).abs().max())
     return rep

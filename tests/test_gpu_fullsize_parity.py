@@ -20,7 +20,7 @@ SUMS_RTOL = 2e-4
 
 
 def _check_heads(w, q, k, r, heads, chunk, use_triton):
-    tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "outside_band": 0}
+    tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "ties": 0, "outside_band": 0}
     for h in heads:
         rep = head_mask_parity(q, k, h, r["mask"][h], w.stride, w.threshold, chunk, w.causal,
                                pad0_quirk=not use_triton, sums_got=r["sums"][h])

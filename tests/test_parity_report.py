@@ -3,7 +3,7 @@ the threshold crossing and tolerate flips at it."""
 import torch
 
 from oracle import xattn_oracle as O
-from oracle.parity import TAU_BAND, head_mask_parity, mask_mismatch_report
+from oracle.parity import TAU_BAND, head_mask_parity, mask_mismatch_detail, mask_mismatch_report
 
 
 def _row_case(causal):
@@ -74,3 +74,56 @@ def test_head_mask_parity_runs_one_head_of_a_grouped_layout():
     _, m2 = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, 8, threshold=taus, chunk_size=256,
                              pad0_quirk=False)
     assert head_mask_parity(q, k, 2, m2[0, 2], 8, taus, 256, True, False)["mismatches"] == 0
+
+
+def test_ties_cut_by_the_crossing_are_excused_only_when_the_counts_agree():
+    # row [5, 1, 1, 1, 1, 1] (total 10), tau 0.65: need 6.5 -> the 5 and two of the five equal blocks are kept;
+    # WHICH two is the sort's business
+    x = torch.tensor([[[5.0, 1.0, 1.0, 1.0, 1.0, 1.0]]])
+    want = O.find_blocks_chunked(x[None], 0, 0.65, None, decoding=False, mode="prefill", causal=False)[0]
+    assert int(want.sum()) == 3 and want[0, 0, 0]
+    got = torch.tensor([[[True, False, False, True, False, True]]])
+    if not torch.equal(got, want):
+        d = mask_mismatch_detail(x, got, want, 0.65, False, 0)
+        assert d["outside"] == 0 and d["ties"] == d["mismatches"] > 0
+    three = torch.tensor([[[True, True, True, True, False, False]]])       # one too many of the run
+    assert mask_mismatch_detail(x, three, want, 0.65, False, 0)["outside"] > 0
+    dropped = want.clone()
+    dropped[0, 0, 0] = False                                                  # the big block is not part of any run
+    assert mask_mismatch_detail(x, dropped, want, 0.65, False, 0)["outside"] == 1
+
+
+def _first_chunk_row(vals, want, got, tau):
+    """One causal q-block row of the first query chunk (the diagonal is the last listed value)."""
+    diag = len(vals) - 1
+    x = torch.zeros(1, diag + 1, 32)
+    x[0, diag, : len(vals)] = torch.tensor(vals)
+    w = torch.zeros(1, diag + 1, 32, dtype=torch.bool)
+    g = w.clone()
+    w[0, diag, : len(want)] = torch.tensor(want).bool()
+    g[0, diag, : len(got)] = torch.tensor(got).bool()
+    return mask_mismatch_detail(x, g, w, tau, True, 0, 32)
+
+
+def test_column_zero_comes_free_with_a_cut_run():
+    """Rows of exactly equal sums (uniform attention of zero-padded queries): in the first query chunk
+    column 0 is set whenever a rank is left out, so a selection that spent one of its picks on column 0
+    shows one block fewer than one that did not; both are outcomes of the reference's unstable sort."""
+    v = [2.12759852] * 7 + [1.10680962]
+    d = _first_chunk_row(v, [1, 1, 1, 1, 1, 1, 0, 1], [1, 1, 1, 1, 1, 0, 0, 1], 0.5)
+    assert d == {"mismatches": 1, "in_band": 0, "ties": 1, "outside": 0}
+    d = _first_chunk_row(v, [1, 1, 1, 1, 1, 1, 0, 1], [1, 1, 1, 1, 0, 0, 0, 1], 0.5)     # two fewer: an error
+    assert d["outside"] == 2
+    d = _first_chunk_row([0.43079475] * 16 + [0.10728443], [1] * 8 + [0] + [1] * 8, [1] * 14 + [0, 0, 1], 0.8)
+    assert d["outside"] == 0 and d["ties"] == 3
+    # the oracle itself lands on one of the allowed outcomes
+    x = torch.zeros(1, 1, 8, 32)
+    x[0, 0, 7, :8] = torch.tensor(v)
+    for r in range(7):
+        x[0, 0, r, : r + 1] = 1.0
+    want = O.find_blocks_chunked(x, 0, 0.5, None, decoding=False, mode="prefill", causal=True)[0]
+    lowest = torch.zeros(32, dtype=torch.bool)
+    lowest[[0, 1, 2, 3, 4, 7]] = True
+    got = want.clone()
+    got[0, 7] = lowest
+    assert mask_mismatch_detail(x[0], got, want, 0.5, True, 0, 32)["outside"] == 0
