@@ -20,8 +20,43 @@ def test_config_rules():
         FastPrefillConfig(threshold=0.9, metric="minfer")
     with pytest.raises(ValueError):
         FastPrefillConfig(threshold=torch.rand(4))
+
+
+def test_default_thresholds_come_from_the_profiled_tables(tmp_path, monkeypatch):
+    """``FastPrefillConfig()`` with no threshold (the reference's default construction,
+    xattn/src/load_llama.py:249-266) reads ``llama_fuse_<stride>``: from the JSON file the
+    profiler writes, or from a module of plain lists put in place of the loader."""
+    import sys
+    import types
+
+    from xattn.src.load_llama import FastPrefillConfig
+    from xattn.threshold import llama_threshold
+
+    monkeypatch.setenv("XATTN_THRESHOLD_TABLES", str(tmp_path / "none.json"))
     with pytest.raises(ValueError, match="llama_threshold"):
-        FastPrefillConfig()          # no tables are shipped
+        FastPrefillConfig()                         # no tables anywhere: the error names where they are looked for
+    g = torch.Generator().manual_seed(0)
+    t16, t8 = torch.rand(32, 32, generator=g), torch.rand(32, 32, generator=g)
+    path = str(tmp_path / "tables.json")
+    llama_threshold.write_tables(path, llama_fuse_16=t16)
+    llama_threshold.write_tables(path, llama_fuse_8=t8.tolist())       # added to the same file
+    monkeypatch.setenv("XATTN_THRESHOLD_TABLES", path)
+    c = FastPrefillConfig()
+    assert c.stride == 16 and c.threshold.shape == (32, 32) and torch.allclose(c.threshold, t16)
+    assert torch.allclose(FastPrefillConfig(stride=8).layer_threshold(12), t8[12])
+    with pytest.raises(ValueError, match="llama_fuse_4"):
+        FastPrefillConfig(stride=4)                 # that stride was never profiled
+    with pytest.raises(ValueError):
+        llama_threshold.write_tables(path, llama_fuse_32=t8)
+    # the reference's module form: plain module-level lists under the same import path
+    stub = types.ModuleType("xattn.threshold.llama_threshold")
+    stub.llama_fuse_16 = [[0.5] * 4] * 3
+    monkeypatch.setitem(sys.modules, "xattn.threshold.llama_threshold", stub)
+    import xattn.threshold as pkg
+
+    monkeypatch.setattr(pkg, "llama_threshold", stub, raising=False)
+    c = FastPrefillConfig()
+    assert c.threshold.shape == (3, 4) and float(c.layer_threshold(2)[1]) == 0.5
 
 
 def test_patch_binds_every_layer_and_checks_head_dim():

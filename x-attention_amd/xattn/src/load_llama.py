@@ -44,11 +44,13 @@ class FastPrefillConfig(dict):
     threshold:  float - one tau for every layer and head;
                 tensor ``[layers, heads]`` - per-layer rows of per-head taus, as
                 produced by the threshold profiler;
-                None - the per-stride tables of a module
-                ``xattn.threshold.llama_threshold`` (``llama_fuse_4/8/16``,
-                nested lists ``[layers][heads]``) if the caller has put one on the
-                import path; the reference ships tables profiled on
-                Llama-3.1-8B-Instruct, this package does not.
+                None - the profiled table of this stride,
+                ``xattn.threshold.llama_threshold.llama_fuse_<stride>``
+                (``[layers][heads]``; load_llama.py:254-261).  That module reads
+                the tables from a JSON file the profiler writes, or can be
+                replaced by the reference's own module of the same name (tables
+                profiled on Llama-3.1-8B-Instruct, parameters of that model,
+                not shipped here); without either it raises ``ValueError``.
     stride:     antidiagonal stride, 4, 8 or 16.
     metric:     "xattn" or "full".
     print_detail: print per-stage wall times (synchronises the device).
@@ -64,13 +66,10 @@ class FastPrefillConfig(dict):
         self.metric = metric
         self.stride = stride
         if threshold is None:
-            try:
-                from xattn.threshold import llama_threshold as tables
-            except ImportError as exc:
-                raise ValueError(
-                    "no threshold given and no module xattn.threshold.llama_threshold on the import path; "
-                    "pass threshold=<float or [layers, heads] tensor>"
-                ) from exc
+            # the profiled [layers, heads] table of this stride (xattn/src/load_llama.py:254-261);
+            # raises ValueError naming where a table is looked for when there is none
+            from xattn.threshold import llama_threshold as tables
+
             threshold = torch.tensor(getattr(tables, f"llama_fuse_{stride}"), dtype=torch.float32)
         if isinstance(threshold, torch.Tensor):
             if threshold.dim() != 2:
@@ -143,7 +142,15 @@ def forward_eval(self, hidden_states, position_embeddings=None, attention_mask=N
             pos = cache_position if cache_position is not None else (position_ids[0] if position_ids is not None else None)
             if pos is None:
                 raise ValueError("a static cache needs cache_position or position_ids to know how much of it is filled")
-            filled = min(int(pos[-1]) + 1, key_states.shape[2])
+            # reading the position costs a device-to-host copy: do it once per model forward (every layer is
+            # handed the same tensor object), not once per layer
+            memo = getattr(cfg, "_filled_memo", None)
+            if memo is not None and memo[0] is pos and memo[1] == pos._version:
+                last = memo[2]
+            else:
+                last = int(pos[-1])
+                cfg._filled_memo = (pos, pos._version, last)
+            filled = min(last + 1, key_states.shape[2])
             key_states, value_states = key_states[:, :, :filled], value_states[:, :, :filled]
     if key_states.device != query_states.device:
         key_states = key_states.to(query_states.device)

@@ -161,6 +161,9 @@ def main():
     parser.add_argument("--texts", type=str, default="xattn/threshold/profile_threshold/text.json",
                         help="JSON list of calibration texts")
     parser.add_argument("--out", type=str, default=None, help="write the table here (torch.save) instead of printing")
+    parser.add_argument("--write-tables", type=str, default=None,
+                        help="add the table as llama_fuse_<stride> to this JSON file, the form "
+                             "xattn.threshold.llama_threshold reads for FastPrefillConfig()")
     args = parser.parse_args()
     model = LlamaForCausalLM.from_pretrained(args.name_or_path, device_map="cuda", torch_dtype=torch.bfloat16).eval()
     tokenizer = AutoTokenizer.from_pretrained(args.name_or_path)
@@ -168,9 +171,13 @@ def main():
         texts = json.load(f)
     batches = (tokenizer(t, return_tensors="pt").input_ids for t in texts)
     table = profile_model(model, ProfileConfig(stride=args.stride), batches)
+    if args.write_tables:
+        from xattn.threshold.llama_threshold import write_tables
+
+        write_tables(args.write_tables, **{f"llama_fuse_{args.stride}": table.float().cpu()})
     if args.out:
         torch.save(table, args.out)
-    else:
+    elif not args.write_tables:
         print(table.tolist())
 
 
