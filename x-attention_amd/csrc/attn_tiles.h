@@ -72,6 +72,7 @@ __host__ __device__ inline DispatchShape dispatch_shape(int H, int Hkv) {
 
 // Returns false for ids that carry no work.
 __host__ __device__ inline bool map_workgroup(int id, int H, int Hkv, int qb_begin, int qb_end, int* head, int* qb) {
+  if (id < 0) return false;
   const DispatchShape d = dispatch_shape(H, Hkv);
   const int x = id & 7, s = id >> 3;
   const int unit = (s / kUnit) * 8 + x, w = s % kUnit;

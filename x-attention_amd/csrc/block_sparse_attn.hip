@@ -40,9 +40,191 @@ struct AttnParams {
   int qb_begin, qb_end;     // q-blocks handled by this launch
   int causal, kv_off;       // kv_off = Lk - Lq
   float scale_log2;         // softmax_scale * log2(e)
+  int* queue;               // persistent form: 8 ticket counters + 1 exit counter (all zero between launches)
+  int queue_len;            // tickets per queue (workgroup ids of the plain launch / 8)
 };
 
 __device__ __forceinline__ int clamp_block(int kb, int nkb) { return kb < 0 ? 0 : (kb < nkb ? kb : nkb - 1); }
+
+// Per-lane addressing that does not depend on the (head, q-block) being worked on.
+struct LaneAddr {
+  int voffK[8], voffV[8];   // tile copy: byte offsets of the lane's rows
+  int kaddr[8];             // K fragment (k-step s, key tile nt): row nt*32 + r, logical chunk 2s + hh
+  int vaddr[4][2];          // V^T fragment (k-step ks, half a, feature tile dt)
+};
+
+__device__ __forceinline__ void lane_addressing(const AttnParams& p, int lane, int wave, LaneAddr& a) {
+  const int r = lane & 31, hh = lane >> 5;
+  tile_offsets(p.k_sn, lane, wave, a.voffK);
+  tile_offsets(p.v_sn, lane, wave, a.voffV);
+#pragma unroll
+  for (int s = 0; s < 8; ++s) a.kaddr[s] = r * 256 + (((2 * s + hh) ^ swz(r)) << 4);
+  // the transposing read hands lane l the feature dt*32 + (l % 32) of keys
+  // 16ks + 8a + 4hh + {0..3}; as a source lane it points at key e = (l%16)/4 of
+  // that quad, features dt*32 + 16*((l/16)%2) + 4*(l%4) .. +3.
+  const int e = (lane & 15) >> 2, j = lane & 3, g2 = (lane >> 4) & 1;
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int row = 8 * h2 + 4 * hh + e;                       // + 16*ks
+      const int c = dt * 4 + 2 * g2 + (j >> 1);
+      a.vaddr[dt][h2] = row * 256 + ((c ^ swz(row)) << 4) + (j & 1) * 8;
+    }
+}
+
+// Q^T fragments of one lane's query row (rows past the end repeat the last one; their output is never stored)
+__device__ __forceinline__ void load_q(const __bf16* qbase, int64_t q_sn, int q_row, int Lq, int hh, bf16x8 (&qreg)[8]) {
+  const int row = q_row < Lq ? q_row : Lq - 1;
+  const __bf16* src = qbase + (int64_t)row * q_sn + hh * 8;
+#pragma unroll
+  for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(src + s * 16);
+}
+
+// S^T = K_j Q^T : lane owns query row r, key rows 8g + 4hh + t of each 32-row tile
+__device__ __forceinline__ void qk_tile(const char* Ks, const int (&kaddr)[8], const bf16x8 (&qreg)[8], f32x16 (&sacc)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) sacc[i][v] = 0.f;
+  bf16x8 kf[2][4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) kf[0][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[0] + nt * 8192);
+  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    if (s < 7) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+        kf[(s + 1) & 1][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[s + 1] + nt * 8192);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) sacc[nt] = mfma32(kf[s & 1][nt], qreg[s], sacc[nt]);
+    if (s < 7) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    } else {
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    }
+  }
+}
+
+// Online softmax in the exp2 domain on the scores of one tile; leaves the bf16
+// probabilities in pfrag (already in the B-operand layout of O^T += V^T P^T).
+// The reference maximum m_run is only moved when a row's maximum outgrows it
+// by more than 2^8 (or on the row's first visible key): exp2 arguments then
+// stay <= 8, which fp32 sums and bf16 probabilities hold without loss, and
+// the rescaling of l and of the 64 output accumulators is skipped for the
+// wavefront whenever no row needs it.  O / l does not depend on the choice.
+__device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[4], f32x16 (&oacc)[4], float& m_run, float& l_run,
+                                             float scale_log2, bf16x8 (&pfrag)[8]) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[nt][v]);
+  mx = fmaxf(mx, swap_half(mx)) * scale_log2;
+  const bool move = mx > m_run + 8.f || (m_run == -INFINITY && mx > -INFINITY);
+  if (__any(move)) {
+    const float m_new = move ? mx : m_run;
+    const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
+    m_run = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+  }
+  const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
+  float psum = 0.f;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float e = fast_exp2(__builtin_fmaf(sacc[nt][v], scale_log2, -m_safe));
+      psum += e;
+      pfrag[nt * 2 + (v >> 3)][v & 7] = (__bf16)e;
+    }
+  l_run += psum;
+}
+
+// O^T += V_j^T P^T
+__device__ __forceinline__ void pv_tile(const char* Vs, const int (&vaddr)[4][2], const bf16x8 (&pfrag)[8], f32x16 (&oacc)[4]) {
+  i16x4 vf[2][4][2];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+      vf[0][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a]));
+  __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    if (ks < 7) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+          vf[(ks + 1) & 1][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a] + (ks + 1) * 4096));
+    }
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+      typedef __attribute__((__vector_size__(8 * sizeof(short)))) short i16x8;
+      i16x8 av;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        av[u] = vf[ks & 1][dt][0][u];
+        av[4 + u] = vf[ks & 1][dt][1][u];
+      }
+      oacc[dt] = mfma32(__builtin_bit_cast(bf16x8, av), pfrag[ks], oacc[dt]);
+    }
+    if (ks < 7) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    } else {
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    }
+  }
+}
+
+// token-level masking of one tile's scores: keys past the sequence end, and (causal) keys after the query
+__device__ __forceinline__ void mask_tile(f32x16 (&sacc)[4], int kb, int hh, int q_pos, int Lk, int causal) {
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int kpos = kb * kBlk + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
+      const bool dead = kpos >= Lk || (causal && kpos > q_pos);
+      sacc[nt][v] = dead ? -INFINITY : sacc[nt][v];
+    }
+}
+
+// normalises and stores this lane's output row
+__device__ __forceinline__ void store_out(const AttnParams& p, int head, int q_row, int hh, const f32x16 (&oacc)[4], float l_run) {
+  const float l_tot = l_run + swap_half(l_run);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (q_row < p.Lq) {
+    __bf16* dst = p.o + (int64_t)head * p.o_sh + (int64_t)q_row * p.o_sn + hh * 4;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = pack_bf16(oacc[dt][g * 4 + 0] * inv, oacc[dt][g * 4 + 1] * inv);
+        w[1] = pack_bf16(oacc[dt][g * 4 + 2] * inv, oacc[dt][g * 4 + 3] * inv);
+        *reinterpret_cast<u32x2*>(dst + dt * 32 + g * 8) = w;
+      }
+  }
+}
+
+typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
 // kHasList = false is the dense baseline (its own symbol, so profiles tell the two apart)
 template <bool kHasList>
@@ -65,7 +247,6 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   int n_blocks;
   // the column list is read through the scalar cache (uniform, read-only), so that
   // fetching the next block id never waits on the tile copies in flight
-  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
   const_i32_ptr list = nullptr;
   {
     const int q_last = (qb * kBlk + kBlk - 1 < p.Lq ? qb * kBlk + kBlk - 1 : p.Lq - 1) + p.kv_off;
@@ -80,39 +261,10 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     }
   }
 
-  // Q^T fragments stay in registers for the whole sweep.
-  bf16x8 qreg[8];
-  {
-    const int row = q_row < p.Lq ? q_row : p.Lq - 1;
-    const __bf16* src = qbase + (int64_t)row * p.q_sn + hh * 8;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(src + s * 16);
-  }
-
-  // loop-invariant addressing
-  int voffK[8], voffV[8];
-  tile_offsets(p.k_sn, lane, wave, voffK);
-  tile_offsets(p.v_sn, lane, wave, voffV);
-  // K fragment (k-step s, key tile nt): row nt*32 + r, logical chunk 2s + hh
-  int kaddr[8];
-#pragma unroll
-  for (int s = 0; s < 8; ++s) kaddr[s] = r * 256 + (((2 * s + hh) ^ swz(r)) << 4);
-  // V^T fragment (k-step ks, half a, feature tile dt): the transposing read hands
-  // lane l the feature dt*32 + (l % 32) of keys 16ks + 8a + 4hh + {0..3}; as a
-  // source lane it points at key e = (l%16)/4 of that quad, features
-  // dt*32 + 16*((l/16)%2) + 4*(l%4) .. +3.
-  int vaddr[4][2];
-  {
-    const int e = (lane & 15) >> 2, j = lane & 3, g2 = (lane >> 4) & 1;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int a = 0; a < 2; ++a) {
-        const int row = 8 * a + 4 * hh + e;                       // + 16*ks
-        const int c = dt * 4 + 2 * g2 + (j >> 1);
-        vaddr[dt][a] = row * 256 + ((c ^ swz(row)) << 4) + (j & 1) * 8;
-      }
-  }
+  bf16x8 qreg[8];   // Q^T fragments stay in registers for the whole sweep
+  load_q(qbase, p.q_sn, q_row, p.Lq, hh, qreg);
+  LaneAddr la;
+  lane_addressing(p, lane, wave, la);
 
   f32x16 oacc[4];
 #pragma unroll
@@ -125,159 +277,208 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   int kb = 0;
   if (n_blocks > 0) {
     kb = kHasList ? clamp_block(list[0], p.nkb) : 0;
-    copy_tile(kbase, p.k_sn, p.Lk, kb, voffK, Ks, wave);
-    copy_tile(vbase, p.v_sn, p.Lk, kb, voffV, Vs, wave);
+    copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
+    copy_tile(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
   }
   wait_vm0();
   __syncthreads();                         // K_0 (and V_0) landed and visible
 
   for (int j = 0; j < n_blocks; ++j) {
     const int kb_next = (j + 1 < n_blocks) ? (kHasList ? clamp_block(list[j + 1], p.nkb) : j + 1) : -1;
-
-    // ---- S^T = K_j Q^T : lane owns query row r, key rows 8g + 4hh + t of each 32-row tile
     f32x16 sacc[4];
+    qk_tile(Ks, la.kaddr, qreg, sacc);
+    wait_vm0();
+    __syncthreads();                       // everyone is done with K_j; V_j landed and visible
+    if (kb_next >= 0) copy_tile(kbase, p.k_sn, p.Lk, kb_next, la.voffK, Ks, wave);
+
+    const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
+    if (need_mask) mask_tile(sacc, kb, hh, q_pos, p.Lk, p.causal);
+    bf16x8 pfrag[8];
+    softmax_tile(sacc, oacc, m_run, l_run, p.scale_log2, pfrag);
+    pv_tile(Vs, la.vaddr, pfrag, oacc);
+    wait_vm0();
+    __syncthreads();                       // everyone is done with V_j; K_{j+1} landed and visible
+    if (kb_next >= 0) copy_tile(vbase, p.v_sn, p.Lk, kb_next, la.voffV, Vs, wave);
+    kb = kb_next;
+  }
+  store_out(p, head, q_row, hh, oacc, l_run);
+}
+
+// ---------------------------------------------------------------------------
+// Persistent form of the list kernel.  512 workgroups (two per CU) stay
+// resident and draw (head, q-block) units from eight ticket queues, one per
+// XCD, holding the units the plain launch would give that XCD in the same
+// order (ticket t of queue x is workgroup id 8t + x of map_workgroup), so an
+// XCD still streams one KV head through its L2; a workgroup whose own queue
+// is exhausted goes on with the next one, which evens out the tail.  The next
+// ticket is drawn while the current unit's first tile is computed; once it is
+// known the next unit's Q rows, first K tile and first V tile are fetched
+// during the current unit's last tile, so a unit switch costs the output
+// store and nothing else - most lists are 2-3 blocks long, where the per-unit
+// start-up of a fresh workgroup (dispatch, count, list head, Q rows, first
+// tiles: ~6 us) is as long as the unit's work.
+// queue[0..7] count the tickets drawn beyond the first 64 of each queue
+// (workgroup b starts with ticket b / 8 of queue b % 8); queue[8] counts
+// finished workgroups and the last one zeroes all nine, so a launch leaves
+// the counters as it found them: zero.
+constexpr int kPersistentGrid = 512;
+constexpr int kQueueSlots = kPersistentGrid / 8;   // first tickets handed out by position
+
+__global__ __launch_bounds__(256, 2) void block_sparse_persistent_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(1024))) char Ks[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) char Vs[kTileBytes];
+  __shared__ int s_ticket;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, hh = lane >> 5;
+  const int group = p.H / p.Hkv;
+  const_i32_ptr cnts = (const_i32_ptr)(uintptr_t)p.col_cnt;
+
+  LaneAddr la;
+  lane_addressing(p, lane, wave, la);
+
+  int queue = blockIdx.x & 7;   // queue currently drawn from
+  int exhausted = 0;            // queues found empty so far (they never refill)
+
+  // Draws tickets, moving on to the next queue when one is exhausted, until a
+  // ticket maps to work.  `first` >= 0 is a ticket already held.  Uniform over
+  // the workgroup; returns false when all eight queues are exhausted.
+  auto acquire = [&](int first, int* head, int* qb) -> bool {
+    for (;;) {
+      int t = first;
+      first = -1;
+      if (t < 0) {
+        if (tid == 0) s_ticket = kQueueSlots + atomicAdd(&p.queue[queue], 1);
+        __syncthreads();
+        t = s_ticket;
+        __syncthreads();
+      }
+      if ((unsigned)t >= (unsigned)p.queue_len) {   // past the end (or counters that were not zero: never index with it)
+        if (++exhausted >= 8) return false;
+        queue = (queue + 1) & 7;
+        continue;
+      }
+      if (map_workgroup(t * 8 + queue, p.H, p.Hkv, p.qb_begin, p.qb_end, head, qb)) return true;
+    }
+  };
+
+  int head = 0, qb = 0;
+  bool have = acquire((int)(blockIdx.x >> 3), &head, &qb);
+
+  bf16x8 qreg[8];
+  f32x16 oacc[4];
+  bool staged = false;          // the current unit's Q rows and first tiles were fetched during the previous unit
+  int n_blocks = 0, kb = 0;
+  const_i32_ptr list = nullptr;
+
+  while (have) {
+    const int kvh = head / group;
+    const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+    const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
+    const int q_row = qb * kBlk + wave * 32 + r;
+    const int q_pos = q_row + p.kv_off;
+    if (!staged) {
+      list = (const_i32_ptr)(uintptr_t)(p.col_idx + ((int64_t)head * p.idx_rows + qb) * p.idx_pitch);
+      n_blocks = cnts[head * p.idx_rows + qb];
+      n_blocks = n_blocks < 0 ? 0 : (n_blocks > p.idx_pitch ? (int)p.idx_pitch : n_blocks);
+      load_q(p.q + (int64_t)head * p.q_sh, p.q_sn, q_row, p.Lq, hh, qreg);
+      if (n_blocks > 0) {
+        kb = clamp_block(list[0], p.nkb);
+        copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
+        copy_tile(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
+      }
+      wait_vm0();
+      __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) sacc[i][v] = 0.f;
-    {
-      bf16x8 kf[2][4];
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) kf[0][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[0] + nt * 8192);
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        if (s < 7) {
-#pragma unroll
-          for (int nt = 0; nt < 4; ++nt)
-            kf[(s + 1) & 1][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[s + 1] + nt * 8192);
-        }
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt) sacc[nt] = mfma32(kf[s & 1][nt], qreg[s], sacc[nt]);
-        if (s < 7) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          }
-        } else {
-          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // the next ticket is drawn now and looked at after the first tile
+    int drawn = -1;
+    if (tid == 0) drawn = atomicAdd(&p.queue[queue], 1);
+    bool next_known = false, next_valid = false;
+    int t_next = 0;                        // the drawn ticket, once every lane knows it
+    int nhead = 0, nqb = 0, n_next = 0, kb_first = 0;
+    const_i32_ptr list_next = nullptr;
+    staged = false;
+
+    for (int j = 0; j < n_blocks; ++j) {
+      const bool last = j + 1 == n_blocks;
+      const int kb_next = last ? -1 : clamp_block(list[j + 1], p.nkb);
+      f32x16 sacc[4];
+      qk_tile(Ks, la.kaddr, qreg, sacc);
+      wait_vm0();
+      __syncthreads();                     // everyone is done with K_j (and with the Q rows when last); V_j landed
+      if (!last) {
+        copy_tile(kbase, p.k_sn, p.Lk, kb_next, la.voffK, Ks, wave);
+      } else if (next_valid) {
+        // unit switch, first half: the next unit's Q rows and first K tile
+        load_q(p.q + (int64_t)nhead * p.q_sh, p.q_sn, nqb * kBlk + wave * 32 + r, p.Lq, hh, qreg);
+        if (n_next > 0)
+          copy_tile(p.k + (int64_t)(nhead / group) * p.k_sh, p.k_sn, p.Lk, kb_first, la.voffK, Ks, wave);
+        staged = true;
+      }
+      if (j == 0 && tid == 0) s_ticket = kQueueSlots + drawn;
+
+      const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
+      if (need_mask) mask_tile(sacc, kb, hh, q_pos, p.Lk, p.causal);
+      bf16x8 pfrag[8];
+      softmax_tile(sacc, oacc, m_run, l_run, p.scale_log2, pfrag);
+      pv_tile(Vs, la.vaddr, pfrag, oacc);
+      wait_vm0();
+      __syncthreads();                     // everyone is done with V_j; K_{j+1} (or the next unit's K_0) landed
+      if (j == 0) {
+        t_next = s_ticket;
+        next_known = true;
+        next_valid = (unsigned)t_next < (unsigned)p.queue_len &&
+                     map_workgroup(t_next * 8 + queue, p.H, p.Hkv, p.qb_begin, p.qb_end, &nhead, &nqb);
+        if (next_valid) {
+          list_next = (const_i32_ptr)(uintptr_t)(p.col_idx + ((int64_t)nhead * p.idx_rows + nqb) * p.idx_pitch);
+          n_next = cnts[nhead * p.idx_rows + nqb];
+          n_next = n_next < 0 ? 0 : (n_next > p.idx_pitch ? (int)p.idx_pitch : n_next);
+          kb_first = n_next > 0 ? clamp_block(list_next[0], p.nkb) : 0;
         }
       }
+      if (!last) copy_tile(vbase, p.v_sn, p.Lk, kb_next, la.voffV, Vs, wave);
+      else if (staged && n_next > 0)       // unit switch, second half: the next unit's first V tile
+        copy_tile(p.v + (int64_t)(nhead / group) * p.v_sh, p.v_sn, p.Lk, kb_first, la.voffV, Vs, wave);
+      kb = kb_next;
     }
-    wait_vm0();
-    __syncthreads();                       // everyone is done with K_j; V_j landed and visible
-    if (kb_next >= 0) copy_tile(kbase, p.k_sn, p.Lk, kb_next, voffK, Ks, wave);
+    store_out(p, head, q_row, hh, oacc, l_run);
 
-    const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
-    if (need_mask) {
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int kpos = kb * kBlk + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
-          const bool dead = kpos >= p.Lk || (p.causal && kpos > q_pos);
-          sacc[nt][v] = dead ? -INFINITY : sacc[nt][v];
-        }
+    if (!next_known) {                     // a unit without tiles: the drawn ticket has not been published yet
+      if (tid == 0) s_ticket = kQueueSlots + drawn;
+      __syncthreads();
+      t_next = s_ticket;
+      __syncthreads();
+      next_valid = (unsigned)t_next < (unsigned)p.queue_len &&
+                   map_workgroup(t_next * 8 + queue, p.H, p.Hkv, p.qb_begin, p.qb_end, &nhead, &nqb);
     }
-
-    // ---- online softmax in the exp2 domain
-    float mx = -INFINITY;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[nt][v]);
-    mx = fmaxf(mx, swap_half(mx)) * p.scale_log2;
-    // The reference maximum m_run is only moved when a row's maximum outgrows it
-    // by more than 2^8 (or on the row's first visible key): exp2 arguments then
-    // stay <= 8, which fp32 sums and bf16 probabilities hold without loss, and
-    // the rescaling of l and of the 64 output accumulators is skipped for the
-    // wavefront whenever no row needs it.  O / l does not depend on the choice.
-    const bool move = mx > m_run + 8.f || (m_run == -INFINITY && mx > -INFINITY);
-    if (__any(move)) {
-      const float m_new = move ? mx : m_run;
-      const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run - m_new);
-      m_run = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
-    }
-    const float m_safe = (m_run == -INFINITY) ? 0.f : m_run;
-    float psum = 0.f;
-    bf16x8 pfrag[8];
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float e = fast_exp2(__builtin_fmaf(sacc[nt][v], p.scale_log2, -m_safe));
-        psum += e;
-        pfrag[nt * 2 + (v >> 3)][v & 7] = (__bf16)e;
+    if (staged) {                          // everything of the next unit is in flight or landed already
+      head = nhead; qb = nqb; n_blocks = n_next; list = list_next; kb = kb_first;
+    } else if (next_valid) {
+      head = nhead; qb = nqb;
+    } else {
+      // the drawn ticket was past the queue's end or a gap in the map: draw again, next queues included
+      if ((unsigned)t_next >= (unsigned)p.queue_len) {
+        if (++exhausted >= 8) break;
+        queue = (queue + 1) & 7;
       }
-    l_run += psum;
-
-    // ---- O^T += V_j^T P^T
-    {
-      i16x4 vf[2][4][2];
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-          vf[0][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a]));
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        if (ks < 7) {
-#pragma unroll
-          for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-              vf[(ks + 1) & 1][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                  (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a] + (ks + 1) * 4096));
-        }
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          typedef __attribute__((__vector_size__(8 * sizeof(short)))) short i16x8;
-          i16x8 av;
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            av[u] = vf[ks & 1][dt][0][u];
-            av[4 + u] = vf[ks & 1][dt][1][u];
-          }
-          oacc[dt] = mfma32(__builtin_bit_cast(bf16x8, av), pfrag[ks], oacc[dt]);
-        }
-        if (ks < 7) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          }
-        } else {
-          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-        }
-      }
+      have = acquire(-1, &head, &qb);
     }
-    wait_vm0();
-    __syncthreads();                       // everyone is done with V_j; K_{j+1} landed and visible
-    if (kb_next >= 0) copy_tile(vbase, p.v_sn, p.Lk, kb_next, voffV, Vs, wave);
-    kb = kb_next;
   }
 
-  const float l_tot = l_run + swap_half(l_run);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (q_row < p.Lq) {
-    __bf16* dst = p.o + (int64_t)head * p.o_sh + (int64_t)q_row * p.o_sn + hh * 4;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack_bf16(oacc[dt][g * 4 + 0] * inv, oacc[dt][g * 4 + 1] * inv);
-        w[1] = pack_bf16(oacc[dt][g * 4 + 2] * inv, oacc[dt][g * 4 + 3] * inv);
-        *reinterpret_cast<u32x2*>(dst + dt * 32 + g * 8) = w;
-      }
+  // the last workgroup out zeroes the counters for the next launch
+  if (tid == 0) {
+    __threadfence();
+    const int done = atomicAdd(&p.queue[8], 1);
+    if (done == (int)gridDim.x - 1) {
+      __threadfence();
+      for (int i = 0; i < 9; ++i) atomicExch(&p.queue[i], 0);
+    }
   }
 }
 
@@ -293,7 +494,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
                                       int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                                       int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
                                       int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,
-                                      int causal, float softmax_scale, void* stream) {
+                                      int causal, float softmax_scale, int32_t* queue, void* stream) {
   if (!q || !k || !v || !out) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
@@ -331,7 +532,13 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   p.qb_end = q_block_end;
   const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
-  if (col_idx)
+  p.queue = queue;
+  p.queue_len = (int)(grid / 8);
+  if (queue && (reinterpret_cast<uintptr_t>(queue) & 3)) return XATTN_ERR_ALIGN;
+  if (col_idx && queue && grid > kPersistentGrid)
+    hipLaunchKernelGGL(block_sparse_persistent_kernel, dim3(kPersistentGrid), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+  else if (col_idx)
     hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
   else
