@@ -160,14 +160,6 @@ int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uin
  * the baseline the speedup is quoted against.  Only query blocks
  * [q_block_begin, q_block_end) are computed (q_block_end < 0: up to the last),
  * so query chunks can be launched as their block lists become available.
- * `queue` (may be null) points at nine int32 in device memory that are ZERO when
- * the launch starts; with it and a column list the launch takes the persistent
- * form: 512 resident workgroups draw (head, q-block) units from ticket counters
- * kept there, which removes the per-unit start-up cost that dominates short
- * lists.  The kernel leaves all nine at zero again, so the same nine ints can
- * serve every later launch ON THE SAME STREAM without being cleared; launches
- * that may run concurrently (other streams) need their own.  Results do not
- * depend on whether a queue is given.
  */
 int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* out,
                            const int32_t* col_idx, const int32_t* col_cnt, int64_t idx_pitch,
@@ -176,7 +168,7 @@ int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* ou
                            int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                            int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
                            int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,
-                           int causal, float softmax_scale, int32_t* queue, void* stream);
+                           int causal, float softmax_scale, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Single-token decode attention over a KV cache.  Replaces the call to the

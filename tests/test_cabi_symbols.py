@@ -58,7 +58,7 @@ def test_attention_entry_points_validate_strides_and_scale_before_launching():
 
     def fwd(strides, scale=0.1, heads=4, kv=2):
         return lib.xattn_block_sparse_fwd(a, a, a, a, None, None, 0, 0, heads, kv, 256, 256, 128, *strides, 0, -1, 1,
-                                          scale, None, None)
+                                          scale, None)
 
     big = 1 << 23
     assert fwd([ok_strides[0], 128, ok_strides[2], big] + ok_strides[4:]) == -4        # K token stride beyond 2^22

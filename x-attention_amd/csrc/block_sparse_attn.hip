@@ -40,8 +40,6 @@ struct AttnParams {
   int qb_begin, qb_end;     // q-blocks handled by this launch
   int causal, kv_off;       // kv_off = Lk - Lq
   float scale_log2;         // softmax_scale * log2(e)
-  int* queue;               // persistent form: 8 ticket counters + 1 exit counter (all zero between launches)
-  int queue_len;            // tickets per queue (workgroup ids of the plain launch / 8)
 };
 
 __device__ __forceinline__ int clamp_block(int kb, int nkb) { return kb < 0 ? 0 : (kb < nkb ? kb : nkb - 1); }
@@ -304,184 +302,6 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   store_out(p, head, q_row, hh, oacc, l_run);
 }
 
-// ---------------------------------------------------------------------------
-// Persistent form of the list kernel.  512 workgroups (two per CU) stay
-// resident and draw (head, q-block) units from eight ticket queues, one per
-// XCD, holding the units the plain launch would give that XCD in the same
-// order (ticket t of queue x is workgroup id 8t + x of map_workgroup), so an
-// XCD still streams one KV head through its L2; a workgroup whose own queue
-// is exhausted goes on with the next one, which evens out the tail.  The next
-// ticket is drawn while the current unit's first tile is computed; once it is
-// known the next unit's Q rows, first K tile and first V tile are fetched
-// during the current unit's last tile, so a unit switch costs the output
-// store and nothing else - most lists are 2-3 blocks long, where the per-unit
-// start-up of a fresh workgroup (dispatch, count, list head, Q rows, first
-// tiles: ~6 us) is as long as the unit's work.
-// queue[0..7] count the tickets drawn beyond the first 64 of each queue
-// (workgroup b starts with ticket b / 8 of queue b % 8); queue[8] counts
-// finished workgroups and the last one zeroes all nine, so a launch leaves
-// the counters as it found them: zero.
-constexpr int kPersistentGrid = 512;
-constexpr int kQueueSlots = kPersistentGrid / 8;   // first tickets handed out by position
-
-__global__ __launch_bounds__(256, 2) void block_sparse_persistent_kernel(AttnParams p) {
-  __shared__ __attribute__((aligned(1024))) char Ks[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) char Vs[kTileBytes];
-  __shared__ int s_ticket;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 31, hh = lane >> 5;
-  const int group = p.H / p.Hkv;
-  const_i32_ptr cnts = (const_i32_ptr)(uintptr_t)p.col_cnt;
-
-  LaneAddr la;
-  lane_addressing(p, lane, wave, la);
-
-  int queue = blockIdx.x & 7;   // queue currently drawn from
-  int exhausted = 0;            // queues found empty so far (they never refill)
-
-  // Draws tickets, moving on to the next queue when one is exhausted, until a
-  // ticket maps to work.  `first` >= 0 is a ticket already held.  Uniform over
-  // the workgroup; returns false when all eight queues are exhausted.
-  auto acquire = [&](int first, int* head, int* qb) -> bool {
-    for (;;) {
-      int t = first;
-      first = -1;
-      if (t < 0) {
-        if (tid == 0) s_ticket = kQueueSlots + atomicAdd(&p.queue[queue], 1);
-        __syncthreads();
-        t = s_ticket;
-        __syncthreads();
-      }
-      if ((unsigned)t >= (unsigned)p.queue_len) {   // past the end (or counters that were not zero: never index with it)
-        if (++exhausted >= 8) return false;
-        queue = (queue + 1) & 7;
-        continue;
-      }
-      if (map_workgroup(t * 8 + queue, p.H, p.Hkv, p.qb_begin, p.qb_end, head, qb)) return true;
-    }
-  };
-
-  int head = 0, qb = 0;
-  bool have = acquire((int)(blockIdx.x >> 3), &head, &qb);
-
-  bf16x8 qreg[8];
-  f32x16 oacc[4];
-  bool staged = false;          // the current unit's Q rows and first tiles were fetched during the previous unit
-  int n_blocks = 0, kb = 0;
-  const_i32_ptr list = nullptr;
-
-  while (have) {
-    const int kvh = head / group;
-    const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
-    const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
-    const int q_row = qb * kBlk + wave * 32 + r;
-    const int q_pos = q_row + p.kv_off;
-    if (!staged) {
-      list = (const_i32_ptr)(uintptr_t)(p.col_idx + ((int64_t)head * p.idx_rows + qb) * p.idx_pitch);
-      n_blocks = cnts[head * p.idx_rows + qb];
-      n_blocks = n_blocks < 0 ? 0 : (n_blocks > p.idx_pitch ? (int)p.idx_pitch : n_blocks);
-      load_q(p.q + (int64_t)head * p.q_sh, p.q_sn, q_row, p.Lq, hh, qreg);
-      if (n_blocks > 0) {
-        kb = clamp_block(list[0], p.nkb);
-        copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
-        copy_tile(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
-      }
-      wait_vm0();
-      __syncthreads();
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-
-    // the next ticket is drawn now and looked at after the first tile
-    int drawn = -1;
-    if (tid == 0) drawn = atomicAdd(&p.queue[queue], 1);
-    bool next_known = false, next_valid = false;
-    int t_next = 0;                        // the drawn ticket, once every lane knows it
-    int nhead = 0, nqb = 0, n_next = 0, kb_first = 0;
-    const_i32_ptr list_next = nullptr;
-    staged = false;
-
-    for (int j = 0; j < n_blocks; ++j) {
-      const bool last = j + 1 == n_blocks;
-      const int kb_next = last ? -1 : clamp_block(list[j + 1], p.nkb);
-      f32x16 sacc[4];
-      qk_tile(Ks, la.kaddr, qreg, sacc);
-      wait_vm0();
-      __syncthreads();                     // everyone is done with K_j (and with the Q rows when last); V_j landed
-      if (!last) {
-        copy_tile(kbase, p.k_sn, p.Lk, kb_next, la.voffK, Ks, wave);
-      } else if (next_valid) {
-        // unit switch, first half: the next unit's Q rows and first K tile
-        load_q(p.q + (int64_t)nhead * p.q_sh, p.q_sn, nqb * kBlk + wave * 32 + r, p.Lq, hh, qreg);
-        if (n_next > 0)
-          copy_tile(p.k + (int64_t)(nhead / group) * p.k_sh, p.k_sn, p.Lk, kb_first, la.voffK, Ks, wave);
-        staged = true;
-      }
-      if (j == 0 && tid == 0) s_ticket = kQueueSlots + drawn;
-
-      const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
-      if (need_mask) mask_tile(sacc, kb, hh, q_pos, p.Lk, p.causal);
-      bf16x8 pfrag[8];
-      softmax_tile(sacc, oacc, m_run, l_run, p.scale_log2, pfrag);
-      pv_tile(Vs, la.vaddr, pfrag, oacc);
-      wait_vm0();
-      __syncthreads();                     // everyone is done with V_j; K_{j+1} (or the next unit's K_0) landed
-      if (j == 0) {
-        t_next = s_ticket;
-        next_known = true;
-        next_valid = (unsigned)t_next < (unsigned)p.queue_len &&
-                     map_workgroup(t_next * 8 + queue, p.H, p.Hkv, p.qb_begin, p.qb_end, &nhead, &nqb);
-        if (next_valid) {
-          list_next = (const_i32_ptr)(uintptr_t)(p.col_idx + ((int64_t)nhead * p.idx_rows + nqb) * p.idx_pitch);
-          n_next = cnts[nhead * p.idx_rows + nqb];
-          n_next = n_next < 0 ? 0 : (n_next > p.idx_pitch ? (int)p.idx_pitch : n_next);
-          kb_first = n_next > 0 ? clamp_block(list_next[0], p.nkb) : 0;
-        }
-      }
-      if (!last) copy_tile(vbase, p.v_sn, p.Lk, kb_next, la.voffV, Vs, wave);
-      else if (staged && n_next > 0)       // unit switch, second half: the next unit's first V tile
-        copy_tile(p.v + (int64_t)(nhead / group) * p.v_sh, p.v_sn, p.Lk, kb_first, la.voffV, Vs, wave);
-      kb = kb_next;
-    }
-    store_out(p, head, q_row, hh, oacc, l_run);
-
-    if (!next_known) {                     // a unit without tiles: the drawn ticket has not been published yet
-      if (tid == 0) s_ticket = kQueueSlots + drawn;
-      __syncthreads();
-      t_next = s_ticket;
-      __syncthreads();
-      next_valid = (unsigned)t_next < (unsigned)p.queue_len &&
-                   map_workgroup(t_next * 8 + queue, p.H, p.Hkv, p.qb_begin, p.qb_end, &nhead, &nqb);
-    }
-    if (staged) {                          // everything of the next unit is in flight or landed already
-      head = nhead; qb = nqb; n_blocks = n_next; list = list_next; kb = kb_first;
-    } else if (next_valid) {
-      head = nhead; qb = nqb;
-    } else {
-      // the drawn ticket was past the queue's end or a gap in the map: draw again, next queues included
-      if ((unsigned)t_next >= (unsigned)p.queue_len) {
-        if (++exhausted >= 8) break;
-        queue = (queue + 1) & 7;
-      }
-      have = acquire(-1, &head, &qb);
-    }
-  }
-
-  // the last workgroup out zeroes the counters for the next launch
-  if (tid == 0) {
-    __threadfence();
-    const int done = atomicAdd(&p.queue[8], 1);
-    if (done == (int)gridDim.x - 1) {
-      __threadfence();
-      for (int i = 0; i < 9; ++i) atomicExch(&p.queue[i], 0);
-    }
-  }
-}
-
 }  // namespace xattn
 
 using namespace xattn;
@@ -494,7 +314,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
                                       int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                                       int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
                                       int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,
-                                      int causal, float softmax_scale, int32_t* queue, void* stream) {
+                                      int causal, float softmax_scale, void* stream) {
   if (!q || !k || !v || !out) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
@@ -532,13 +352,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   p.qb_end = q_block_end;
   const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
-  p.queue = queue;
-  p.queue_len = (int)(grid / 8);
-  if (queue && (reinterpret_cast<uintptr_t>(queue) & 3)) return XATTN_ERR_ALIGN;
-  if (col_idx && queue && grid > kPersistentGrid)
-    hipLaunchKernelGGL(block_sparse_persistent_kernel, dim3(kPersistentGrid), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), p);
-  else if (col_idx)
+  if (col_idx)
     hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
   else

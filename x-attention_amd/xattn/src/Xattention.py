@@ -301,25 +301,8 @@ def xattn_estimate(
     return attn_sums, simple_masks
 
 
-_queues = {}
-
-
-def _queue_for(dev, stream):
-    """Ticket counters of the persistent attention launch: nine zeroed int32 per
-    (device, stream), allocated once - the kernel leaves them at zero, and
-    launches on one stream cannot overlap.  The zero fill is enqueued on the
-    very stream that will use the counters, so the first launch cannot run
-    ahead of it."""
-    stream = stream if stream is not None else torch.cuda.current_stream(dev)
-    key = (dev.index, int(stream.cuda_stream))
-    if key not in _queues:
-        with torch.cuda.stream(stream):
-            _queues[key] = torch.zeros(16, dtype=torch.int32, device=dev)
-    return _queues[key].data_ptr()
-
-
 def block_sparse_attention(query_states, key_states, value_states, col_idx=None, col_cnt=None,
-                           causal=True, softmax_scale=None, out=None, q_blocks=None, stream=None, persistent=True):
+                           causal=True, softmax_scale=None, out=None, q_blocks=None, stream=None):
     """Attention of each 128-token query block over the key blocks listed for it
     (``col_idx``/``col_cnt`` as written by :func:`estimate_and_select`; ``None``
     visits every visible block = dense FlashAttention).  Stands in for
@@ -327,8 +310,6 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
     Returns ``[1, H, q_len, 128]`` as a transposed view of ``[1, q_len, H, 128]``.
     ``out`` (a ``[1, q_len, H, 128]`` buffer), ``q_blocks=(begin, end)`` and ``stream``
     (a ``torch.cuda.Stream``) let a caller fill the output chunk by chunk.
-    ``persistent=False`` launches one workgroup per (head, q-block) instead of
-    512 resident ones drawing units from a queue (same result, for comparison).
     """
     lib = _hb.lib()
     q = _check_qk(query_states, "query_states")
@@ -366,7 +347,7 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
                 pitch, idx_rows, heads, kv_heads, q_len, k_len, 128,
                 q.stride(1), q.stride(2), k.stride(1), k.stride(2), v.stride(1), v.stride(2),
                 out.stride(2), out.stride(1), qb0, qb1, int(bool(causal)), scale,
-                _queue_for(dev, stream) if (col_idx is not None and persistent) else None, stream_ptr,
+                stream_ptr,
             ),
             "xattn_block_sparse_fwd",
         )

@@ -41,7 +41,7 @@ _SIGNATURES = {
     ),
     "xattn_block_sparse_fwd": (
         c_i32,
-        [c_vp] * 6 + [c_i64] + [c_i32] * 6 + [c_i64] * 8 + [c_i32, c_i32, c_i32, c_f32, c_vp, c_vp],
+        [c_vp] * 6 + [c_i64] + [c_i32] * 6 + [c_i64] * 8 + [c_i32, c_i32, c_i32, c_f32, c_vp],
     ),
 }
 
