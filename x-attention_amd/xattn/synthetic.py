@@ -86,8 +86,16 @@ def _ar1(x, dim, rho):
     return x
 
 
-def make_inputs(w: Workload, device="cpu", seed=0, L=None, heads=None, kv_heads=None, dtype=None):
-    """q [1,H,L,128], k, v [1,H_kv,L,128] for a workload (optionally shrunk)."""
+def make_inputs(w: Workload, device="cpu", seed=0, L=None, heads=None, kv_heads=None, dtype=None, rank8="head"):
+    """q [1,H,L,128], k, v [1,H_kv,L,128] for a workload (optionally shrunk).
+
+    ``rank8`` chooses the reading of the text workloads' "shared rank-8 Gaussian
+    component": "head" (default) is the per-KV-head direction described above;
+    "token" draws a coefficient vector c_t ~ N(0, I_8) per TOKEN instead and adds
+    ``2.0 * c_t B / sqrt(8)`` to that token's query (every head) and key (every
+    KV head) - shared between q and k of a token, not along the sequence, which
+    gives diffuse attention without locality (kept as the dense end of the
+    benchmark's density sweep)."""
     L = w.L if L is None else L
     H = w.heads if heads is None else heads
     Hkv = w.kv_heads if kv_heads is None else kv_heads
@@ -127,14 +135,17 @@ def make_inputs(w: Workload, device="cpu", seed=0, L=None, heads=None, kv_heads=
     if w.kind == "video+text":
         frames = 240 if L == w.L else max(1, (L * 240 // w.L))
         n_video = min(L, frames * 256)
+    if rank8 not in ("head", "token"):
+        raise ValueError("rank8 must be 'head' or 'token'")
     coeff = _randn((Hkv, 8), gen, device)
     basis = _randn((8, D), gen, device)
     direction = 2.0 * (coeff @ basis) / math.sqrt(8.0)   # [Hkv, D], rank 8, shared by q and k
+    per_token = 2.0 * (_randn((L, 8), gen, device) @ basis) / math.sqrt(8.0) if rank8 == "token" else None
 
     def tokens(kv_head, shared):
         x = _randn((L, D), gen, device)
         if shared:
-            x[n_video:] += direction[kv_head]
+            x[n_video:] += direction[kv_head] if per_token is None else per_token[n_video:]
         if n_video:
             nf = (n_video + 255) // 256
             means = _randn((nf, D), gen, device).repeat_interleave(256, dim=0)[:n_video]
