@@ -196,7 +196,7 @@ def density_sweep(w, L, chunk, dev, t_dense, qkv, steps=3):
         for tau in taus:
             for i in range(steps + 1):
                 marks = []
-                r = estimate_and_select(q, k, w.stride, tau, chunk, causal=True, marks=marks)
+                r = estimate_and_select(q, k, w.stride, tau, chunk, causal=True, marks=marks, want_mask=False)
                 block_sparse_attention(q, k, v, r["col_idx"], r["col_cnt"], causal=True)
                 end = torch.cuda.Event(enable_timing=True)
                 end.record()
@@ -269,7 +269,8 @@ def main():
     torch.cuda.synchronize()
 
     def step(marks=None):
-        r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, marks=marks)
+        # what the operator itself runs: column lists only, no byte mask
+        r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, marks=marks, want_mask=False)
         if marks is not None:
             marks.append(("sparse_begin", marks[-1][1]))
         out = block_sparse_attention(q, k, v, r["col_idx"], r["col_cnt"], causal=w.causal)
@@ -383,6 +384,7 @@ def main():
 
         kept = r["col_cnt"].long().sum(-1)
         heads = sorted({int(kept.argmin()), int(kept.argmax())})
+        r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, want_lists=False)     # with the mask
         tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "ties": 0, "outside_band": 0}
         for h in heads:
             rep = head_mask_parity(q, k, h, r["mask"][h], w.stride, tau, chunk, w.causal, pad0_quirk=False)

@@ -96,6 +96,12 @@ const char* xattn_error_string(int code);
  * their position on the key axis instead (xattn/src/kernels.py:70 with the
  * real_q_len of Xattention.py:169): n_rq - (k_len_padded - k_len)/stride; padded
  * query rows that rule leaves alone carry the uniform softmax of a zero query.
+ * window_row0 / window_rows: block_sums may hold only the q-block rows
+ * [window_row0, window_row0 + window_rows) of every head, laid out
+ * [num_heads][window_rows][k_len_padded/block_size] (row i of the result at row
+ * i - window_row0); the chunks of the call must lie inside the window.
+ * window_rows <= 0 means the whole padded result.  A caller that works through
+ * a long sequence in groups of query chunks needs buffers for one group only.
  * `workspace` must hold xattn_estimate_workspace_bytes(...) bytes, where
  * chunks_per_call is the largest chunk_end - chunk_begin used (<= 0: all chunks);
  * the function returns 0 for arguments the estimator rejects.
@@ -109,7 +115,8 @@ int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, v
                               int64_t q_stride_n, int64_t k_stride_h, int64_t k_stride_n, int stride,
                               int block_size, int chunk_size, int chunk_begin, int chunk_end, int causal,
                               int own_chunk_only, float scale, const int32_t* slab_pairs,
-                              int num_slab_pairs, int softmax, int kdb, int zero_rows_from, void* stream);
+                              int num_slab_pairs, int softmax, int kdb, int zero_rows_from, int window_row0,
+                              int window_rows, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Threshold block selection.  Replaces find_blocks_chunked,
@@ -138,13 +145,19 @@ int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, v
  *          col_idx [H][nq_blocks][idx_pitch] ascending kept columns that are
  *          < list_cols and, when causal, hold a key visible to the row's last
  *          query token given kv_off_tokens = k_len - q_len;  col_cnt [H][nq_blocks].
- * col_idx/col_cnt may both be null.  nk_blocks <= 16384.
+ * col_idx/col_cnt may both be null; so may mask when the lists are asked for
+ * (the operator itself only needs the lists).  nk_blocks <= 16384.
+ * window_row0 / window_rows: block_sums, mask, col_idx and col_cnt hold the
+ * q-block rows [window_row0, window_row0 + window_rows) of every head (row i at
+ * row i - window_row0; per-head pitch window_rows rows); [row_begin, row_end)
+ * must lie inside.  window_rows <= 0 means all nq_blocks rows.
  */
 int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uint8_t* mask,
                         int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int num_heads,
                         int nq_blocks, int nk_blocks, int row_begin, int row_end, int diag_offset,
                         int causal, int keep_sink, int keep_recent, int list_cols, int q_len,
-                        int kv_off_tokens, int blocks_per_chunk, void* stream);
+                        int kv_off_tokens, int blocks_per_chunk, int window_row0, int window_rows,
+                        void* stream);
 
 /* ---------------------------------------------------------------------------
  * Block-sparse FlashAttention forward.  Replaces the call
@@ -153,8 +166,10 @@ int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uin
  *                          is_causal=causal)      xattn/src/Xattention.py:377-391
  * for one sequence (cu_seqlens = [0, len]) and per-head masks.  Query block
  * qb (128 tokens) of head h visits the col_cnt[h][qb] key blocks listed in
- * col_idx[h][qb][*] (arrays of idx_rows >= ceil(q_len/128) rows per head, each
- * idx_pitch entries long, as xattn_select_blocks writes them); inside a block, when causal, key c is visible to query t
+ * col_idx[h][qb - idx_row0][*] (arrays of idx_rows rows per head holding the
+ * q-blocks [idx_row0, idx_row0 + idx_rows), each row idx_pitch entries long, as
+ * xattn_select_blocks writes them; the q-blocks of the launch must lie inside);
+ * inside a block, when causal, key c is visible to query t
  * iff c <= t + (k_len - q_len).  A query row with no visible key yields zeros.
  * col_idx == col_cnt == null visits every visible block: dense FlashAttention,
  * the baseline the speedup is quoted against.  Only query blocks
@@ -163,8 +178,8 @@ int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uin
  */
 int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* out,
                            const int32_t* col_idx, const int32_t* col_cnt, int64_t idx_pitch,
-                           int idx_rows, int num_heads, int num_kv_heads, int q_len, int k_len,
-                           int head_dim,
+                           int idx_rows, int idx_row0, int num_heads, int num_kv_heads, int q_len,
+                           int k_len, int head_dim,
                            int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                            int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
                            int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,

@@ -57,7 +57,7 @@ def test_attention_entry_points_validate_strides_and_scale_before_launching():
     ok_strides = [128 * 256, 128, 128 * 256, 128, 128 * 256, 128, 128, 128 * 4]
 
     def fwd(strides, scale=0.1, heads=4, kv=2):
-        return lib.xattn_block_sparse_fwd(a, a, a, a, None, None, 0, 0, heads, kv, 256, 256, 128, *strides, 0, -1, 1,
+        return lib.xattn_block_sparse_fwd(a, a, a, a, None, None, 0, 0, 0, heads, kv, 256, 256, 128, *strides, 0, -1, 1,
                                           scale, None)
 
     big = 1 << 23

@@ -30,7 +30,7 @@ def _select(sums, tau, causal, diag_offset, keep_sink=False, keep_recent=False):
         lib.xattn_select_blocks(
             s.data_ptr(), t.data_ptr(), mask.data_ptr(), idx.data_ptr(), cnt.data_ptr(), nk,
             H, nq, nk, 0, nq, diag_offset, int(causal), int(keep_sink), int(keep_recent),
-            nk, nq * 128, diag_offset * 128, nq, torch.cuda.current_stream().cuda_stream,
+            nk, nq * 128, diag_offset * 128, nq, 0, 0, torch.cuda.current_stream().cuda_stream,
         ),
         "xattn_select_blocks",
     )

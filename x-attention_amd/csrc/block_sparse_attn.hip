@@ -35,7 +35,8 @@ struct AttnParams {
   const int32_t* col_idx;   // [H, idx_rows, idx_pitch] ascending k-block ids, or null = all visible
   const int32_t* col_cnt;   // [H, idx_rows]
   int64_t idx_pitch;
-  int idx_rows;             // q-block rows per head in col_idx / col_cnt (>= nqb)
+  int idx_rows;             // q-block rows per head in col_idx / col_cnt
+  int idx_row0;             // q-block held by their row 0
   int H, Hkv, Lq, Lk, nqb, nkb;
   int qb_begin, qb_end;     // q-blocks handled by this launch
   int causal, kv_off;       // kv_off = Lk - Lq
@@ -251,8 +252,9 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     int visible = p.causal ? (q_last < 0 ? 0 : q_last / kBlk + 1) : p.nkb;
     visible = visible < p.nkb ? visible : p.nkb;
     if (kHasList) {
-      list = (const_i32_ptr)(uintptr_t)(p.col_idx + ((int64_t)head * p.idx_rows + qb) * p.idx_pitch);
-      n_blocks = ((const_i32_ptr)(uintptr_t)p.col_cnt)[head * p.idx_rows + qb];
+      const int64_t slot = (int64_t)head * p.idx_rows + (qb - p.idx_row0);
+      list = (const_i32_ptr)(uintptr_t)(p.col_idx + slot * p.idx_pitch);
+      n_blocks = ((const_i32_ptr)(uintptr_t)p.col_cnt)[slot];
       n_blocks = n_blocks < 0 ? 0 : (n_blocks > p.idx_pitch ? (int)p.idx_pitch : n_blocks);
     } else {
       n_blocks = visible;
@@ -310,7 +312,8 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* out,
                                       const int32_t* col_idx, const int32_t* col_cnt, int64_t idx_pitch,
-                                      int idx_rows, int num_heads, int num_kv_heads, int q_len, int k_len, int head_dim,
+                                      int idx_rows, int idx_row0, int num_heads, int num_kv_heads, int q_len, int k_len,
+                                      int head_dim,
                                       int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
                                       int64_t k_stride_n, int64_t v_stride_h, int64_t v_stride_n,
                                       int64_t o_stride_h, int64_t o_stride_n, int q_block_begin, int q_block_end,
@@ -343,11 +346,13 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   p.causal = causal ? 1 : 0;
   p.kv_off = k_len - q_len;
   p.scale_log2 = softmax_scale * kLog2e;
-  if (col_idx && (idx_pitch < 1 || idx_rows < p.nqb)) return XATTN_ERR_SHAPE;
-  p.idx_rows = idx_rows;
-
   if (q_block_end < 0) q_block_end = p.nqb;
   if (q_block_begin < 0 || q_block_begin >= q_block_end || q_block_end > p.nqb) return XATTN_ERR_SHAPE;
+  // the lists may hold a window of q-block rows only; the q-blocks of this launch must lie inside it
+  if (col_idx && (idx_pitch < 1 || idx_row0 < 0 || q_block_begin < idx_row0 || q_block_end > idx_row0 + idx_rows))
+    return XATTN_ERR_SHAPE;
+  p.idx_rows = idx_rows;
+  p.idx_row0 = idx_row0;
   p.qb_begin = q_block_begin;
   p.qb_end = q_block_end;
   const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);

@@ -38,7 +38,8 @@ struct EstParams {
   float* Mt;       // [H][nT][rows]   tile maximum (exp2 domain)
   float* Lt;       // [H][nT][rows]   tile sum
   float* scores;   // optional [H][n_rq][n_rk] raw scores
-  float* sums;     // [H][nqb][nkb] output block sums
+  float* sums;     // output block sums: [H][win_rows][nkb], q-block row i stored at row i - win_row0
+  int win_row0, win_rows;
   int H, Hkv, Lq, Lk, S, rbs;
   int n_rq, n_rk, nkb, nqb, nT;
   int rcs;                  // reshaped keys per chunk
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
   int hi4 = row_hi(p, mc4);
   hi4 = hi4 < p.n_rk - 1 ? hi4 : p.n_rk - 1;
   const int kb_hi = hi4 / RBS;
-  float* out = p.sums + ((int64_t)head * p.nqb + mc4 / RBS) * p.nkb;
+  float* out = p.sums + ((int64_t)head * p.win_rows + (mc4 / RBS - p.win_row0)) * p.nkb;
   constexpr int kLanesPerBlock = RBS / 4;          // lanes whose 4-row sums make up one query block
   int T_cached = -1;
   f32x4 wgt = {0.f, 0.f, 0.f, 0.f};
@@ -492,7 +493,7 @@ __global__ __launch_bounds__(256) void estimate_normalize_rows_kernel(EstParams 
     rowInv[row] = real ? (p.no_softmax ? 1.f : 1.f / Lr) : 0.f;
   }
   __syncthreads();
-  float* out = p.sums + ((int64_t)head * p.nqb + m0 / p.rbs_q) * p.nkb;
+  float* out = p.sums + ((int64_t)head * p.win_rows + (m0 / p.rbs_q - p.win_row0)) * p.nkb;
   for (int kb = tid; kb < p.nkb; kb += 256) {
     const int T = (kb * p.rbs) / kSub;
     float acc = 0.f;
@@ -568,7 +569,8 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
                                          int64_t k_stride_n, int stride, int block_size, int chunk_size,
                                          int chunk_begin, int chunk_end, int causal, int own_chunk_only,
                                          float scale, const int32_t* slab_pairs, int num_slab_pairs,
-                                         int softmax, int kdb, int zero_rows_from, void* stream) {
+                                         int softmax, int kdb, int zero_rows_from, int window_row0,
+                                         int window_rows, void* stream) {
   if (!q || !k || !block_sums || !workspace) return XATTN_ERR_NULL;
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
@@ -616,6 +618,15 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.n_pairs = num_slab_pairs;
   p.scores = scores_out;
   p.sums = block_sums;
+  // block_sums may hold a window of q-block rows only; the chunks of this call must lie inside it
+  {
+    const int bpc = chunk_size / block_size;
+    if (window_rows <= 0) { window_row0 = 0; window_rows = g.nqb; }
+    if (window_row0 < 0 || chunk_begin * bpc < window_row0 || chunk_end * bpc > window_row0 + window_rows)
+      return XATTN_ERR_SHAPE;
+    p.win_row0 = window_row0;
+    p.win_rows = window_rows;
+  }
   if (workspace_size < workspace_bytes(num_heads, g, p.rows)) return XATTN_ERR_WORKSPACE;
   float* ws = static_cast<float*>(workspace);
   p.P = ws;

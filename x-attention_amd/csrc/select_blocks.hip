@@ -27,6 +27,7 @@ struct SelParams {
   int32_t* col_cnt;
   int64_t idx_pitch;
   int H, nqb, nkb, row_begin, row_end, diag_offset;
+  int win_row0, win_rows;   // the arrays hold q-block rows [win_row0, win_row0 + win_rows) of every head
   int causal, keep_sink, keep_recent, list_cols, q_len, kv_off;
   int blocks_per_chunk;
   int npow2;   // LDS key capacity (power of two >= nkb)
@@ -56,7 +57,8 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   const int rows = p.row_end - p.row_begin;
   const int head = blockIdx.x / rows;
   const int row = p.row_begin + blockIdx.x % rows;
-  const float* x = p.sums + ((int64_t)head * p.nqb + row) * p.nkb;
+  const int64_t slot = (int64_t)head * p.win_rows + (row - p.win_row0);   // this row's place in the arrays
+  const float* x = p.sums + slot * p.nkb;
   const int diag = row + p.diag_offset;
   // Column index of the first diagonal of the row's query chunk.  When it is 0
   // the reference's eye() assignment overwrites the forced sink column
@@ -213,11 +215,13 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     for (int c = lane; c < p.nkb; c += 64) flags[c] = 1;
   __syncthreads();
 
-  uint8_t* mrow = p.mask + ((int64_t)head * p.nqb + row) * p.nkb;
-  for (int c = lane; c < p.nkb; c += 64) mrow[c] = flags[c];
+  if (p.mask) {
+    uint8_t* mrow = p.mask + slot * p.nkb;
+    for (int c = lane; c < p.nkb; c += 64) mrow[c] = flags[c];
+  }
 
   if (p.col_idx) {
-    int32_t* list = p.col_idx + ((int64_t)head * p.nqb + row) * p.idx_pitch;
+    int32_t* list = p.col_idx + slot * p.idx_pitch;
     const int q_last = (row * 128 + 127 < p.q_len ? row * 128 + 127 : p.q_len - 1) + p.kv_off;
     int count = 0;
     for (int c0 = 0; c0 < p.nkb; c0 += 64) {
@@ -229,7 +233,7 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
       if (keep && pos < p.idx_pitch) list[pos] = c;
       count += __popcll(ballot);
     }
-    if (lane == 0) p.col_cnt[head * p.nqb + row] = count < p.idx_pitch ? count : (int)p.idx_pitch;
+    if (lane == 0) p.col_cnt[slot] = count < p.idx_pitch ? count : (int)p.idx_pitch;
   }
 }
 
@@ -242,9 +246,10 @@ extern "C" int xattn_select_blocks(const float* block_sums, const double* tau_pe
                                    int nq_blocks, int nk_blocks, int row_begin, int row_end,
                                    int diag_offset, int causal, int keep_sink, int keep_recent,
                                    int list_cols, int q_len, int kv_off_tokens, int blocks_per_chunk,
-                                   void* stream) {
-  if (!block_sums || !tau_per_head || !mask) return XATTN_ERR_NULL;
+                                   int window_row0, int window_rows, void* stream) {
+  if (!block_sums || !tau_per_head) return XATTN_ERR_NULL;
   if ((col_idx == nullptr) != (col_cnt == nullptr)) return XATTN_ERR_NULL;
+  if (!mask && !col_idx) return XATTN_ERR_NULL;     // nothing to write
   if (num_heads <= 0 || nq_blocks <= 0 || nk_blocks <= 0 || nk_blocks > 16384) return XATTN_ERR_SHAPE;
   if (row_begin < 0 || row_end > nq_blocks || row_begin >= row_end) return XATTN_ERR_SHAPE;
   if (col_idx && idx_pitch < 1) return XATTN_ERR_SHAPE;
@@ -256,6 +261,9 @@ extern "C" int xattn_select_blocks(const float* block_sums, const double* tau_pe
   p.causal = causal ? 1 : 0; p.keep_sink = keep_sink ? 1 : 0; p.keep_recent = keep_recent ? 1 : 0;
   p.list_cols = list_cols; p.q_len = q_len; p.kv_off = kv_off_tokens;
   p.blocks_per_chunk = blocks_per_chunk;
+  if (window_rows <= 0) { window_row0 = 0; window_rows = nq_blocks; }
+  if (window_row0 < 0 || row_begin < window_row0 || row_end > window_row0 + window_rows) return XATTN_ERR_SHAPE;
+  p.win_row0 = window_row0; p.win_rows = window_rows;
   int np2 = 64;
   while (np2 < nk_blocks) np2 <<= 1;
   p.npow2 = np2;

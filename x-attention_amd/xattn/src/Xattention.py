@@ -27,7 +27,8 @@ from . import hip_backend as _hb
 __all__ = ["Xattention_prefill", "xattn_estimate", "default_chunk_size", "estimate_and_select", "block_sparse_attention"]
 
 BLOCK = 128
-WORKSPACE_LIMIT = 4 << 30   # bytes of estimator workspace per launch
+WORKSPACE_LIMIT = 2 << 30   # bytes of estimator workspace per launch
+GROUP_LIMIT = 2 << 30       # bytes of block sums + column lists the operator holds at a time
 
 
 def default_chunk_size(k_len):
@@ -101,7 +102,8 @@ class _Plan:
     """Geometry, buffers and kernel launchers of one estimate -> select pass."""
 
     def __init__(self, query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs=None, softmax=True, kdb=1):
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs=None, softmax=True, kdb=1,
+                 want_mask=True, group_limit=None):
         self.lib = _hb.lib()
         self.kdb = int(kdb)
         self.softmax = bool(softmax)
@@ -166,20 +168,41 @@ class _Plan:
         self.chunks_per_call = max(1, min(self.q_chunks, WORKSPACE_LIMIT // per_chunk))
         self.ws_bytes = self.lib.xattn_estimate_workspace_bytes(
             self.heads, self.q_len, self.k_len, stride, block_size, chunk_size, self.chunks_per_call)
+        # Block sums, mask and column lists hold a window of q-block rows: all of them, or - when a byte
+        # limit is given and they would exceed it - one group of whole query chunks at a time, which the
+        # caller works through with window(); the buffers are reused from group to group.
+        per_row = self.heads * (self.nkb * 4 + (self.nkb if want_mask else 0)
+                                + ((self.list_cols + 1) * 4 if want_lists else 0))
+        self.chunks_per_group = self.q_chunks
+        if group_limit is not None and per_row * self.nqb > group_limit:
+            self.chunks_per_group = max(1, min(self.q_chunks, group_limit // (per_row * self.blocks_per_chunk)))
+        self.win_rows = self.chunks_per_group * self.blocks_per_chunk
+        self.win_row0 = 0
         with torch.cuda.device(dev):
             self.workspace = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
-            self.sums = torch.empty((self.heads, self.nqb, self.nkb), dtype=torch.float32, device=dev)
+            self.sums = torch.empty((self.heads, self.win_rows, self.nkb), dtype=torch.float32, device=dev)
             self.scores = None
             if dump_scores:
                 self.scores = torch.zeros(
                     (self.heads, (self.q_len + q_pad) // stride // self.kdb, (self.k_len + k_pad) // stride),
                     dtype=torch.float32, device=dev)
             self.tau = _tau_per_head(threshold, self.heads, dev)
-            self.mask = torch.empty((self.heads, self.nqb, self.nkb), dtype=torch.uint8, device=dev)
+            self.mask = None
+            if want_mask:
+                self.mask = torch.empty((self.heads, self.win_rows, self.nkb), dtype=torch.uint8, device=dev)
             self.col_idx = self.col_cnt = None
             if want_lists:
-                self.col_idx = torch.empty((self.heads, self.nqb, self.list_cols), dtype=torch.int32, device=dev)
-                self.col_cnt = torch.empty((self.heads, self.nqb), dtype=torch.int32, device=dev)
+                self.col_idx = torch.empty((self.heads, self.win_rows, self.list_cols), dtype=torch.int32, device=dev)
+                self.col_cnt = torch.empty((self.heads, self.win_rows), dtype=torch.int32, device=dev)
+
+    def groups(self):
+        """(first chunk, end chunk) of every group of query chunks the buffers can hold."""
+        return [(c, min(self.q_chunks, c + self.chunks_per_group))
+                for c in range(0, self.q_chunks, self.chunks_per_group)]
+
+    def window(self, chunk_begin):
+        """Points the buffers at the group of query chunks that starts at ``chunk_begin``."""
+        self.win_row0 = chunk_begin * self.blocks_per_chunk
 
     def estimate(self, chunk_begin, chunk_end, stream):
         if chunk_end - chunk_begin > self.chunks_per_call:
@@ -195,7 +218,7 @@ class _Plan:
                 q.stride(1), q.stride(2), k.stride(1), k.stride(2),
                 self.stride, self.block_size, self.chunk_size, chunk_begin, chunk_end,
                 int(self.causal), int(self.own_chunk_only), self.scale, self.pairs, self.n_pairs,
-                int(self.softmax), self.kdb, self.zero_rows_from, stream,
+                int(self.softmax), self.kdb, self.zero_rows_from, self.win_row0, self.win_rows, stream,
             ),
             "xattn_estimate_block_sums",
         )
@@ -204,11 +227,12 @@ class _Plan:
         lists = self.col_idx is not None
         _hb.check(
             self.lib.xattn_select_blocks(
-                self.sums.data_ptr(), self.tau.data_ptr(), self.mask.data_ptr(),
+                self.sums.data_ptr(), self.tau.data_ptr(), self.mask.data_ptr() if self.mask is not None else None,
                 self.col_idx.data_ptr() if lists else None, self.col_cnt.data_ptr() if lists else None,
                 self.list_cols, self.heads, self.nqb, self.nkb, row_begin, row_end, self.nkb - self.nqb,
                 int(self.causal), int(self.keep_sink), int(self.keep_recent),
-                self.list_cols, self.q_len, self.k_len - self.q_len, self.blocks_per_chunk, stream,
+                self.list_cols, self.q_len, self.k_len - self.q_len, self.blocks_per_chunk,
+                self.win_row0, self.win_rows, stream,
             ),
             "xattn_select_blocks",
         )
@@ -236,19 +260,22 @@ def estimate_and_select(
     slab_pairs=None,
     softmax=True,
     kdb=1,
+    want_mask=True,
 ):
     """Runs the estimator and selection kernels over all query chunks, one launch each.
 
     Returns a dict with fp32 ``sums`` [H, Nq_p, Nk_p], uint8 ``mask`` of the same
     shape, and (when ``want_lists``) ``col_idx`` [H, Nq_p, pitch] / ``col_cnt``
-    [H, Nq_p] for :func:`block_sparse_attention`.
+    [H, Nq_p] for :func:`block_sparse_attention` (``want_mask=False`` skips the
+    byte mask, which the attention kernel does not read).
 
     ``marks``, when a list, receives ``(label, torch.cuda.Event)`` pairs recorded
     on the current stream before the estimator, between estimator and selection
     and after selection (for per-kernel timing).
     """
     plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs, softmax, kdb)
+                 keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs, softmax, kdb,
+                 want_mask=want_mask)
     with torch.cuda.device(plan.dev):
         stream = _stream_ptr(plan.dev)
         _mark(marks, "estimate_begin")
@@ -302,14 +329,16 @@ def xattn_estimate(
 
 
 def block_sparse_attention(query_states, key_states, value_states, col_idx=None, col_cnt=None,
-                           causal=True, softmax_scale=None, out=None, q_blocks=None, stream=None):
+                           causal=True, softmax_scale=None, out=None, q_blocks=None, stream=None, idx_row0=0):
     """Attention of each 128-token query block over the key blocks listed for it
     (``col_idx``/``col_cnt`` as written by :func:`estimate_and_select`; ``None``
     visits every visible block = dense FlashAttention).  Stands in for
     ``block_sparse_attn_func`` at xattn/src/Xattention.py:377-391.
     Returns ``[1, H, q_len, 128]`` as a transposed view of ``[1, q_len, H, 128]``.
     ``out`` (a ``[1, q_len, H, 128]`` buffer), ``q_blocks=(begin, end)`` and ``stream``
-    (a ``torch.cuda.Stream``) let a caller fill the output chunk by chunk.
+    (a ``torch.cuda.Stream``) let a caller fill the output chunk by chunk;
+    ``idx_row0`` says which q-block row 0 of ``col_idx``/``col_cnt`` holds when
+    the lists cover a window of q-blocks only.
     """
     lib = _hb.lib()
     q = _check_qk(query_states, "query_states")
@@ -335,6 +364,8 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
         assert col_idx.is_contiguous() and col_cnt.is_contiguous()
         assert col_idx.shape[0] == heads and col_cnt.shape == col_idx.shape[:2]
         pitch, idx_rows = col_idx.shape[2], col_idx.shape[1]
+        if q_blocks is None:
+            qb0, qb1 = idx_row0, min((q_len + 127) // 128, idx_row0 + idx_rows)
     else:
         pitch, idx_rows = 0, 0
     with torch.cuda.device(dev):
@@ -344,7 +375,7 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                 col_idx.data_ptr() if col_idx is not None else None,
                 col_cnt.data_ptr() if col_cnt is not None else None,
-                pitch, idx_rows, heads, kv_heads, q_len, k_len, 128,
+                pitch, idx_rows, idx_row0, heads, kv_heads, q_len, k_len, 128,
                 q.stride(1), q.stride(2), k.stride(1), k.stride(2), v.stride(1), v.stride(2),
                 out.stride(2), out.stride(1), qb0, qb1, int(bool(causal)), scale,
                 stream_ptr,
@@ -383,14 +414,27 @@ def Xattention_prefill(
     if pipeline_chunks:
         return _prefill_pipelined(query_states, key_states, value_states, stride, norm, threshold, block_size,
                                   use_triton, causal, chunk_size, keep_sink, keep_recent, kdb)
-    r = estimate_and_select(
-        query_states, key_states, stride, threshold, chunk_size, causal=causal, norm=norm,
-        use_triton=use_triton, keep_sink=keep_sink, keep_recent=keep_recent, block_size=block_size,
-        want_lists=True, kdb=kdb,
-    )
-    return block_sparse_attention(
-        query_states, key_states, value_states, r["col_idx"], r["col_cnt"], causal=causal
-    )
+    # One launch per stage when the block sums and column lists of the whole sequence fit GROUP_LIMIT
+    # (128k tokens: 0.26 GB); longer sequences go through the three stages one group of query chunks at a
+    # time on buffers of one group, so the extra memory stays bounded however long the sequence is.
+    plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
+                 keep_sink, keep_recent, block_size, True, False, kdb=kdb, want_mask=False, group_limit=GROUP_LIMIT)
+    dev = plan.dev
+    v = _check_qk(value_states, "value_states")
+    nb = (plan.q_len + block_size - 1) // block_size
+    with torch.cuda.device(dev):
+        stream = _stream_ptr(dev)
+        out = torch.empty((1, plan.q_len, plan.heads, 128), dtype=torch.bfloat16, device=dev)
+        bpc = plan.blocks_per_chunk
+        for c0, c1 in plan.groups():
+            plan.window(c0)
+            plan.estimate(c0, c1, stream)
+            plan.select(c0 * bpc, c1 * bpc, stream)
+            qb0, qb1 = c0 * bpc, min(nb, c1 * bpc)
+            if qb0 < qb1:
+                block_sparse_attention(plan.q, plan.k, v, plan.col_idx, plan.col_cnt, causal=causal, out=out,
+                                       q_blocks=(qb0, qb1), idx_row0=plan.win_row0)
+    return out.transpose(1, 2)
 
 
 _side_streams = {}

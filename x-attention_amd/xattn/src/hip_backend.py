@@ -19,11 +19,11 @@ _SIGNATURES = {
     "xattn_estimate_block_sums": (
         c_i32,
         [c_vp, c_vp, c_vp, c_vp, c_sz, c_vp] + [c_i32] * 5 + [c_i64] * 4 + [c_i32] * 7
-        + [c_f32, ctypes.POINTER(c_i32), c_i32, c_i32, c_i32, c_i32, c_vp],
+        + [c_f32, ctypes.POINTER(c_i32), c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     ),
     "xattn_select_blocks": (
         c_i32,
-        [c_vp] * 5 + [c_i64] + [c_i32] * 13 + [c_vp],
+        [c_vp] * 5 + [c_i64] + [c_i32] * 15 + [c_vp],
     ),
     "xattn_calibration_copy": (c_i32, [c_vp, c_vp, c_sz, c_vp]),
     "xattn_mfma_rate_probe": (c_i32, [c_vp, c_i32, c_vp, ctypes.POINTER(ctypes.c_double), c_vp]),
@@ -41,7 +41,7 @@ _SIGNATURES = {
     ),
     "xattn_block_sparse_fwd": (
         c_i32,
-        [c_vp] * 6 + [c_i64] + [c_i32] * 6 + [c_i64] * 8 + [c_i32, c_i32, c_i32, c_f32, c_vp],
+        [c_vp] * 6 + [c_i64] + [c_i32] * 7 + [c_i64] * 8 + [c_i32, c_i32, c_i32, c_f32, c_vp],
     ),
 }
 

@@ -54,7 +54,7 @@ def flat_group_gemm_fuse_reshape(query_states, key_states, stride, chunk_start, 
                 heads, kv_heads, q_len, k_used.shape[2], 128,
                 q.stride(1), q.stride(2), k_used.stride(1), k_used.stride(2),
                 stride, 128, chunk, 0, q_len // chunk, int(bool(is_causal)), 0,
-                1.0 / math.sqrt(128) / stride, None, 0, 1, 1, -1, _stream_ptr(q.device),
+                1.0 / math.sqrt(128) / stride, None, 0, 1, 1, -1, 0, 0, _stream_ptr(q.device),
             ),
             "xattn_estimate_block_sums",
         )

@@ -44,7 +44,7 @@ def find_blocks_chunked(input_tensor, current_index, threshold, num_to_choose, d
             lib.xattn_select_blocks(
                 sums.data_ptr(), tau.data_ptr(), mask.data_ptr(), None, None, 0,
                 heads, rows, cols, 0, rows, int(current_index), int(bool(causal)), 0, 0,
-                cols, rows * 128, int(current_index) * 128, rows, torch.cuda.current_stream(dev).cuda_stream,
+                cols, rows * 128, int(current_index) * 128, rows, 0, 0, torch.cuda.current_stream(dev).cuda_stream,
             ),
             "xattn_select_blocks",
         )
