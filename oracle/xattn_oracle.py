@@ -111,6 +111,23 @@ def reshape_operands(query_states, key_states, stride, select_mode="inverse", pe
     raise ValueError(select_mode)
 
 
+def create_causal_mask(batch_size, head_num, block_size, block_num, divide_block_num, device="cpu"):
+    """Additive mask of query block ``divide_block_num`` against all key blocks,
+    xattn/src/utils.py:3-42 (the reference hard-codes ``device="cuda"``)."""
+    divide_block_num += 1
+    if divide_block_num < 1 or divide_block_num > block_num:
+        raise ValueError(f"divide_block_num ({divide_block_num}) must be between 1 and block_num ({block_num}).")
+    total = block_size * block_num
+    mask = torch.zeros(block_size, total, device=device)
+    if divide_block_num < block_num:
+        mask[:, divide_block_num * block_size :] = NEG_INF
+    start = (divide_block_num - 1) * block_size
+    mask[:, start : start + block_size] = torch.triu(
+        torch.full((block_size, block_size), NEG_INF, device=device), diagonal=1
+    )
+    return mask[None, None].expand(batch_size, head_num, block_size, total)
+
+
 def antidiagonal_scores(query_states, key_states, stride):
     """score[m, n] = sum_i Q[m*S + S-1-i] . K[n*S + i]  (un-scaled).
 
@@ -150,7 +167,13 @@ def find_blocks_chunked(
     if mode == "prefill" and decoding:
         return torch.ones_like(input_tensor, dtype=torch.bool)
     if mode == "decode" and not decoding:
-        raise NotImplementedError("decode-mode masks are outside the prefill path")
+        # xattn/src/utils.py:71-86, literally: the causal branch joins ROW slices along the column axis
+        ones = torch.ones_like(input_tensor, dtype=torch.bool)
+        if not causal:
+            return ones
+        return torch.cat(
+            [ones[:, :, 0 : current_index + 1], torch.zeros_like(ones)[:, :, current_index + 1 :]], dim=-1
+        )
     dev = input_tensor.device
     x = input_tensor.to(torch.float64)
 

@@ -132,3 +132,37 @@ def test_per_head_threshold_broadcast():
             x[:, h : h + 1], 0, float(taus[h].double()), None, decoding=False, mode="prefill", causal=False
         )
         assert torch.equal(m[:, h : h + 1], mh)
+
+
+def test_create_causal_mask_against_a_loop_and_the_product_helper():
+    """xattn/src/utils.py:3-42: row r of block d sees every earlier block and columns <= r of its own."""
+    from xattn.src.utils import create_causal_mask
+
+    for bs, nb, d in [(4, 3, 0), (4, 3, 1), (4, 3, 2), (8, 1, 0), (2, 5, 3)]:
+        m = O.create_causal_mask(2, 3, bs, nb, d)
+        assert m.shape == (2, 3, bs, bs * nb)
+        for r in range(bs):
+            for c in range(bs * nb):
+                want = 0.0 if c <= d * bs + r else float("-inf")
+                assert m[1, 2, r, c].item() == want, (bs, nb, d, r, c)
+        assert torch.equal(create_causal_mask(2, 3, bs, nb, d, device="cpu"), m)
+    for bad in (-1, 3):
+        with pytest.raises(ValueError):
+            O.create_causal_mask(1, 1, 4, 3, bad)
+        with pytest.raises(ValueError):
+            create_causal_mask(1, 1, 4, 3, bad, device="cpu")
+
+
+def test_decode_mode_of_find_blocks_chunked():
+    """xattn/src/utils.py:71-86: no selection; the causal form is a join of row slices along the
+    column axis, which has a shape only when the slices have equally many rows."""
+    from xattn.src.utils import find_blocks_chunked
+
+    x = torch.rand(1, 2, 4, 6)
+    for f in (O.find_blocks_chunked, find_blocks_chunked):
+        assert f(x, 1, 0.9, None, decoding=False, mode="decode", causal=False).all()
+        m = f(x, 1, 0.9, None, decoding=False, mode="decode", causal=True)       # rows 0..1 | rows 2..3
+        assert m.shape == (1, 2, 2, 12) and m[..., :6].all() and not m[..., 6:].any()
+        with pytest.raises(RuntimeError):
+            f(x, 0, 0.9, None, decoding=False, mode="decode", causal=True)         # 1 row against 3
+        assert f(x, 0, 0.9, None, decoding=True, mode="prefill").all()
