@@ -125,7 +125,7 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[4], f32x16 (&oacc)[4
   for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[nt][v]);
-  mx = fmaxf(mx, swap_half(mx)) * scale_log2;
+  mx = half_max(mx) * scale_log2;
   const bool move = mx > m_run + 8.f || (m_run == -INFINITY && mx > -INFINITY);
   if (__any(move)) {
     const float m_new = move ? mx : m_run;
@@ -207,7 +207,7 @@ __device__ __forceinline__ void mask_tile(f32x16 (&sacc)[4], int kb, int hh, int
 
 // normalises and stores this lane's output row
 __device__ __forceinline__ void store_out(const AttnParams& p, int head, int q_row, int hh, const f32x16 (&oacc)[4], float l_run) {
-  const float l_tot = l_run + swap_half(l_run);
+  const float l_tot = half_sum(l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (q_row < p.Lq) {
     __bf16* dst = p.o + (int64_t)head * p.o_sh + (int64_t)q_row * p.o_sn + hh * 4;

@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256, 1) void decode_partial_kernel(DecodeParams p) 
     float mx = -INFINITY;
 #pragma unroll
     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[v]);
-    mx = fmaxf(mx, swap_half(mx)) * p.scale_log2;
+    mx = half_max(mx) * p.scale_log2;
     const float m_new = fmaxf(m_run, mx);          // finite: every tile holds at least one real key
     const float alpha = fast_exp2(m_run - m_new);  // 0 on the first tile
     m_run = m_new;
@@ -264,7 +264,7 @@ __global__ __launch_bounds__(256, 1) void decode_partial_kernel(DecodeParams p) 
 
   // The four wavefronts' results meet in LDS (each uses the start of its own,
   // now idle, ring) and leave as one partial result per workgroup.
-  const float l_tot = l_run + swap_half(l_run);
+  const float l_tot = half_sum(l_run);
   float* mine = reinterpret_cast<float*>(ring);
   if (r < p.group) {
     float* dst = mine + r * kPartStride;

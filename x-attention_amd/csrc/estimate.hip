@@ -306,7 +306,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
           mx = fmaxf(mx, vis ? acc[nt][mt][v] * p.scale_log2 : -INFINITY);
         }
     }
-    mx = fmaxf(mx, swap_half(mx));
+    mx = half_max(mx);
     const float safe = (mx == -INFINITY) ? 0.f : mx;
     float tot = 0.f;
     const int mrel = m - p.row_begin;
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
           }
           s += e;
         }
-        part[g] = s + swap_half(s);
+        part[g] = half_sum(s);
         tot += part[g];
       }
       // part[g] covers keys nbase + nt*32 + 8g .. +7

@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void block_mass_kernel(MassParams p) {
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[nt][v]);
-      mx = fmaxf(mx, swap_half(mx)) * p.scale_log2;
+      mx = half_max(mx) * p.scale_log2;
       const float m_new = fmaxf(m_run, mx);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       float psum = 0.f;
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256, 2) void block_mass_kernel(MassParams p) {
       l_run = l_run * ((m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_safe)) + psum;
       m_run = m_new;
       if (jj == visible - 1) {
-        const float l_tot = l_run + swap_half(l_run);
+        const float l_tot = half_sum(l_run);
         inv_l = (row_ok && l_tot > 0.f) ? 1.f / l_tot : 0.f;   // padded rows carry no mass
       }
     } else {

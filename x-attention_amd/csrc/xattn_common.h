@@ -40,4 +40,28 @@ __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70);
 // value held by the lane 32 positions away (the other half-wave)
 __device__ __forceinline__ float swap_half(float x) { return __shfl_xor(x, 32, 64); }
 
+// x combined with the value of the lane 32 positions away, in every lane.  One
+// v_permlane32_swap exchanges the upper half of its first operand with the lower
+// half of its second: fed two copies of x it leaves (lower half, lower half) in
+// the first and (upper half, upper half) in the second - both partners in every
+// lane, without a trip through the LDS crossbar.  Written as inline assembly
+// (the compiler's builtin hands back the first result twice); the s_nop pairs
+// cover the wait states the instruction needs after a VALU write of its
+// operands and before a VALU read of its results.
+__device__ __forceinline__ void half_pair(float x, float& lo, float& hi) {
+  lo = x;
+  hi = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float half_sum(float x) {
+  float lo, hi;
+  half_pair(x, lo, hi);
+  return lo + hi;
+}
+__device__ __forceinline__ float half_max(float x) {
+  float lo, hi;
+  half_pair(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+
 }  // namespace xattn
