@@ -148,8 +148,9 @@ def decode_leg(q, k, v, reps=50):
 
 
 def mfma_probe(dev):
-    """What a stream of bf16 MFMAs alone sustains on this part: with constant operand bits and with
-    random ones (the clock the part holds depends on the switching activity of the operands)."""
+    """What a stream of bf16 MFMAs sustains on this part: alone, and with the vector-ALU load of an attention
+    tile (one exponential and three fmas per MFMA, no dependences, no memory) issued beside it; each with constant
+    operand bits and with random ones (the clock the part holds depends on the switching activity of the operands)."""
     import ctypes
 
     import torch
@@ -165,16 +166,17 @@ def mfma_probe(dev):
     }
     for name, host in tables.items():
         bits = host.to(dev)
-        flops = ctypes.c_double(0.0)
-        stream = torch.cuda.current_stream().cuda_stream
-        hip_backend.check(lib.xattn_mfma_rate_probe(bits.data_ptr(), 20000, sink.data_ptr(), ctypes.byref(flops), stream), "probe")
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        hip_backend.check(lib.xattn_mfma_rate_probe(bits.data_ptr(), 100000, sink.data_ptr(), ctypes.byref(flops), stream), "probe")
-        e1.record()
-        torch.cuda.synchronize()
-        res[name + "_tflops"] = round(flops.value / (_ms(e0, e1) * 1e-3) / 1e12, 1)
+        for mix, suffix in ((0, ""), (1, "_with_softmax_valu_mix")):
+            flops = ctypes.c_double(0.0)
+            stream = torch.cuda.current_stream().cuda_stream
+            hip_backend.check(lib.xattn_mfma_rate_probe(bits.data_ptr(), 20000, mix, sink.data_ptr(), ctypes.byref(flops), stream), "probe")
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            hip_backend.check(lib.xattn_mfma_rate_probe(bits.data_ptr(), 100000, mix, sink.data_ptr(), ctypes.byref(flops), stream), "probe")
+            e1.record()
+            torch.cuda.synchronize()
+            res[name + suffix + "_tflops"] = round(flops.value / (_ms(e0, e1) * 1e-3) / 1e12, 1)
     return res
 
 

@@ -286,10 +286,15 @@ int xattn_calibration_copy(void* dst, const void* src, size_t bytes, void* strea
  * floating-point operations of the launch is written to *flops_out (host, may
  * be null); the caller times the launch.  Equal bits everywhere measure the
  * data-independent rate, random bits the rate the part sustains at the
- * switching activity of real inputs.  `sink` is one float of device memory that
- * is practically never written.
+ * switching activity of real inputs.  With valu_mix != 0 every MFMA is
+ * accompanied by one v_exp_f32 and three v_fma_f32 on unrelated registers (the
+ * vector-ALU load per MFMA of the attention tile loop, with no dependences and
+ * no memory traffic): the rate then is what the SIMD's instruction issue
+ * leaves of the MFMA stream under that mix.  `sink` is one float of device
+ * memory that is practically never written.
  */
-int xattn_mfma_rate_probe(const void* operand_bits, int iters, float* sink, double* flops_out, void* stream);
+int xattn_mfma_rate_probe(const void* operand_bits, int iters, int valu_mix, float* sink, double* flops_out,
+                          void* stream);
 
 #ifdef __cplusplus
 }

@@ -20,6 +20,13 @@ __global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* __re
 // differs between the two.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 probe_bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float probe_f32x16;
+// kMix: beside every MFMA the wavefront also issues one v_exp_f32 and three
+// v_fma_f32 on registers no MFMA touches and with no dependence on it - the
+// per-MFMA vector-ALU load of the attention tile loop (64 MFMAs, 65
+// exponentials and about 190 other VALU instructions per tile and wavefront)
+// with every wait taken away.  Its rate is what the SIMD's issue logic leaves
+// of the MFMA stream under that mix, an upper bound for an attention kernel.
+template <bool kMix>
 __global__ __launch_bounds__(256) void mfma_rate_probe_kernel(const probe_bf16x8* __restrict__ bits, int iters,
                                                               float* sink) {
   probe_bf16x8 a[8], b[8];
@@ -33,23 +40,40 @@ __global__ __launch_bounds__(256) void mfma_rate_probe_kernel(const probe_bf16x8
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+  float ex[8], fm[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    ex[e] = (float)a[e][0] * 0.01f;
+    fm[e] = (float)b[e][0];
+  }
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 4; ++i) {
         acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(u * 4 + i) & 7], b[(u + i) & 7], acc[i], 0, 0, 0);
+        if (kMix) {
+          const int j = (u * 4 + i) & 7;
+          ex[j] = __builtin_fmaf(__builtin_amdgcn_exp2f(ex[j]), 0.5f, 0.01f);
+          fm[j] = __builtin_fmaf(fm[j], 0.999f, 0.5f);
+          fm[(j + 4) & 7] = __builtin_fmaf(fm[(j + 4) & 7], 0.998f, 0.25f);
+        }
+      }
   }
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) s += acc[i][v];
-  if (s == 12345.678f) sink[0] = s;   // keeps the accumulators live; practically never taken
+  if (kMix) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += ex[e] + fm[e];
+  }
+  if (s == 12345.678f) sink[0] = s;   // keeps the results live; practically never taken
 }
 }  // namespace xattn
 
-extern "C" int xattn_abi_version(void) { return 5; }
+extern "C" int xattn_abi_version(void) { return 6; }
 
 extern "C" const char* xattn_error_string(int code) {
   switch (code) {
@@ -76,14 +100,18 @@ extern "C" int xattn_calibration_copy(void* dst, const void* src, size_t bytes, 
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
 }
 
-extern "C" int xattn_mfma_rate_probe(const void* operand_bits, int iters, float* sink, double* flops_out,
-                                     void* stream) {
+extern "C" int xattn_mfma_rate_probe(const void* operand_bits, int iters, int valu_mix, float* sink,
+                                     double* flops_out, void* stream) {
   if (!operand_bits || !sink) return XATTN_ERR_NULL;
   if (iters <= 0 || iters > (1 << 22)) return XATTN_ERR_SHAPE;
   if (reinterpret_cast<uintptr_t>(operand_bits) & 15) return XATTN_ERR_ALIGN;
   const int grid = 256 * 2;   // two workgroups of four wavefronts per CU: two wavefronts per SIMD
   if (flops_out) *flops_out = (double)grid * 4.0 * iters * 16.0 * 32768.0;
-  hipLaunchKernelGGL(xattn::mfma_rate_probe_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const xattn::probe_bf16x8*>(operand_bits), iters, sink);
+  if (valu_mix)
+    hipLaunchKernelGGL(xattn::mfma_rate_probe_kernel<true>, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const xattn::probe_bf16x8*>(operand_bits), iters, sink);
+  else
+    hipLaunchKernelGGL(xattn::mfma_rate_probe_kernel<false>, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const xattn::probe_bf16x8*>(operand_bits), iters, sink);
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
 }

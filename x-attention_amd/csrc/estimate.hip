@@ -425,26 +425,36 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
   const int kb_hi = hi4 / RBS;
   float* out = p.sums + ((int64_t)head * p.win_rows + (mc4 / RBS - p.win_row0)) * p.nkb;
   constexpr int kLanesPerBlock = RBS / 4;          // lanes whose 4-row sums make up one query block
-  int T_cached = -1;
-  f32x4 wgt = {0.f, 0.f, 0.f, 0.f};
-  for (int kb0 = wave * 4; kb0 < p.nkb; kb0 += 16) {
-    const int kb = kb0 + kgrp;
-    float acc = 0.f;
-    if (rows_ok && kb < p.nkb && kb >= kb_lo && kb <= kb_hi) {
-      const int T = (kb * RBS) / kSub;
-      if (T != T_cached) {
-        const f32x4 mt = *reinterpret_cast<const f32x4*>(Mst + (int64_t)T * p.rows + mrel4);
+  // Four trips' worth of loads are issued before any of them is used, so that each wavefront keeps four
+  // 16-byte loads in flight instead of one (the pass is bound by memory latency times loads in flight).
+  // A 128-key tile holds 128 / RBS key blocks, so consecutive trips (16 key blocks apart) change tile
+  // unless RBS is 8: the tile weights are recomputed per trip (one load of four tile maxima, four exp2).
+  constexpr int kUnroll = 4;
+  for (int kb0 = wave * 4; kb0 < p.nkb; kb0 += 16 * kUnroll) {
+    f32x4 pv[kUnroll], mt[kUnroll];
+    bool live[kUnroll];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) wgt[i] = fast_exp2(mt[i] - rM[i]) * rI[i];
-        T_cached = T;
+    for (int u = 0; u < kUnroll; ++u) {
+      const int kb = kb0 + 16 * u + kgrp;
+      live[u] = rows_ok && kb < p.nkb && kb >= kb_lo && kb <= kb_hi;
+      if (live[u]) {
+        const int T = (kb * RBS) / kSub;
+        mt[u] = *reinterpret_cast<const f32x4*>(Mst + (int64_t)T * p.rows + mrel4);
+        pv[u] = *reinterpret_cast<const f32x4*>(Pst + (int64_t)kb * p.rows + mrel4);
       }
-      const f32x4 pv = *reinterpret_cast<const f32x4*>(Pst + (int64_t)kb * p.rows + mrel4);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc += (rI[i] != 0.f) ? pv[i] * wgt[i] : 0.f;
     }
 #pragma unroll
-    for (int d = 1; d < kLanesPerBlock; d <<= 1) acc += __shfl_xor(acc, d, 64);
-    if (rows_ok && kb < p.nkb && (l16 % kLanesPerBlock) == 0) out[kb] = acc;
+    for (int u = 0; u < kUnroll; ++u) {
+      const int kb = kb0 + 16 * u + kgrp;
+      float acc = 0.f;
+      if (live[u]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc += (rI[i] != 0.f) ? pv[u][i] * (fast_exp2(mt[u][i] - rM[i]) * rI[i]) : 0.f;
+      }
+#pragma unroll
+      for (int d = 1; d < kLanesPerBlock; d <<= 1) acc += __shfl_xor(acc, d, 64);
+      if (rows_ok && kb < p.nkb && (l16 % kLanesPerBlock) == 0) out[kb] = acc;
+    }
   }
 }
 

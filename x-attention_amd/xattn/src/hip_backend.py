@@ -26,7 +26,7 @@ _SIGNATURES = {
         [c_vp] * 5 + [c_i64] + [c_i32] * 15 + [c_vp],
     ),
     "xattn_calibration_copy": (c_i32, [c_vp, c_vp, c_sz, c_vp]),
-    "xattn_mfma_rate_probe": (c_i32, [c_vp, c_i32, c_vp, ctypes.POINTER(ctypes.c_double), c_vp]),
+    "xattn_mfma_rate_probe": (c_i32, [c_vp, c_i32, c_i32, c_vp, ctypes.POINTER(ctypes.c_double), c_vp]),
     "xattn_softmax_block_sums": (c_i32, [c_vp, c_vp] + [c_i32] * 3 + [c_i64] * 2 + [c_i32] * 3 + [c_f32, c_i32, c_vp]),
     "xattn_block_mass": (c_i32, [c_vp] * 3 + [c_i32] * 5 + [c_i64] * 4 + [c_i32, c_f32, c_vp]),
     "xattn_threshold_rows": (c_i32, [c_vp] * 3 + [c_i32] * 3 + [c_i64] * 2 + [c_f32, c_vp]),
