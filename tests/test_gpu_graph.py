@@ -1,5 +1,6 @@
-"""GPU: the decode step and the block-sparse attention launch are capturable
-in a HIP graph (nothing is allocated or synchronised inside the entry points):
+"""GPU: the decode step, the block-sparse attention launch and the whole
+prefill operator are capturable in a HIP graph (nothing is allocated or
+synchronised inside the entry points, and the operator never reads back):
 every replay, with new contents in the same buffers and eager work in
 between, must reproduce the eager result bit for bit."""
 import pytest
@@ -55,3 +56,29 @@ def test_block_sparse_attention_replays_from_a_graph():
         want = block_sparse_attention(q, k, v, r["col_idx"], r["col_cnt"])
         torch.cuda.synchronize()
         assert torch.equal(got.transpose(1, 2), want), i
+
+
+def test_whole_operator_replays_from_a_graph():
+    """estimate -> select -> attention captured as one graph (temporaries from the
+    capture's memory pool): the selection changes with the inputs from replay
+    to replay, and every replay equals the eager call."""
+    from xattn.src.Xattention import Xattention_prefill
+    from xattn.synthetic import WORKLOADS, make_inputs
+
+    w = WORKLOADS[1]
+    q, k, v = make_inputs(w, device="cuda", seed=3, L=4096 + 200, heads=8, kv_heads=2)
+    kw = dict(threshold=0.9, chunk_size=2048)
+    Xattention_prefill(q, k, v, 8, **kw)                                      # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = Xattention_prefill(q, k, v, 8, **kw)
+    for i in range(3):
+        q2, k2, v2 = make_inputs(w, device="cuda", seed=10 + i, L=4096 + 200, heads=8, kv_heads=2)
+        q.copy_(q2), k.copy_(k2), v.copy_(v2)                                 # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = Xattention_prefill(q, k, v, 8, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), i

@@ -427,8 +427,8 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
   constexpr int kLanesPerBlock = RBS / 4;          // lanes whose 4-row sums make up one query block
   // Four trips' worth of loads are issued before any of them is used, so that each wavefront keeps four
   // 16-byte loads in flight instead of one (the pass is bound by memory latency times loads in flight).
-  // A 128-key tile holds 128 / RBS key blocks, so consecutive trips (16 key blocks apart) change tile
-  // unless RBS is 8: the tile weights are recomputed per trip (one load of four tile maxima, four exp2).
+  // A 128-key tile holds 128 / RBS <= 16 key blocks and consecutive trips are 16 key blocks apart, so every
+  // trip lies in another tile: its weights are computed per trip (one load of four tile maxima, four exp2).
   constexpr int kUnroll = 4;
   for (int kb0 = wave * 4; kb0 < p.nkb; kb0 += 16 * kUnroll) {
     f32x4 pv[kUnroll], mt[kUnroll];
