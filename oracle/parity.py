@@ -11,7 +11,7 @@ from . import xattn_oracle as O
 TAU_BAND = 1e-5      # masks may differ only on blocks whose cumulative mass is this close to tau
 
 
-def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None):
+def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None, keep_recent=False):
     """Compares two block masks given the block sums both were selected from.
 
     Returns a dict: ``mismatches``; ``in_band`` - mismatching blocks for which the
@@ -26,7 +26,10 @@ def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_c
     reference uses torch.sort, xattn/src/utils.py:110,126,150) or, for sums that
     differ in the last bits, the order rounding gives;
     ``outside`` - everything else, i.e. real disagreements.  Forced blocks and
-    blocks beyond the diagonal are never excused.
+    blocks beyond the diagonal are never excused.  ``keep_recent`` says that the
+    masks were post-processed with the block diagonal forced
+    (xattn/src/Xattention.py:288-297): without causality that column is an ordinary
+    candidate of the selection that ends up set whether chosen or not, like column 0.
     """
     import numpy as np
 
@@ -73,11 +76,12 @@ def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_c
         cut = 0 < kept < len(run)
         if cut:
             # any `kept` members of the run may be the chosen ones; column 0, when it is a member, is set
-            # anyway (unselected ranks scatter to it), so a mask may show one chosen member fewer beside it
-            rest = run[run != 0]
-            free0 = len(rest) != len(run)
-            counts = {kept - 1, kept} if free0 else {kept}
-            ok = all(int(m[h, i][rest].sum()) in counts and (not free0 or bool(m[h, i][0])) for m in (got, want))
+            # anyway (unselected ranks scatter to it), and so is the diagonal under keep_recent: a mask may
+            # show one chosen member fewer beside each such member
+            free = [c for c in ([0, diag] if keep_recent and not causal else [0]) if c in run]
+            rest = run[~np.isin(run, free)]
+            counts = set(range(kept - len(free), kept + 1))
+            ok = all(int(m[h, i][rest].sum()) in counts and all(bool(m[h, i][c]) for c in free) for m in (got, want))
             if ok:
                 ties += 1
                 continue
@@ -85,10 +89,10 @@ def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_c
     return {"mismatches": len(bad), "in_band": len(bad) - outside - ties, "ties": ties, "outside": outside}
 
 
-def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None):
+def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_chunk=None, keep_recent=False):
     """(number of mismatching blocks, number of them that the parity contract does
     not excuse) - see :func:`mask_mismatch_detail`."""
-    d = mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_chunk)
+    d = mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_chunk, keep_recent)
     return d["mismatches"], d["outside"]
 
 

@@ -243,3 +243,20 @@ def test_ragged_kv_longer_than_q_follows_each_branch_row_rule(Lq, Lk, C, causal,
     nq_p, nk_p = want_mask.shape[2], want_mask.shape[3]
     nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, causal, nk_p - nq_p, C // 128)
     assert outside == 0, (nbad, outside)
+
+
+@pytest.mark.parametrize("use_triton", [True, False])
+@pytest.mark.parametrize("S,L,C", [(16, 2426, 128), (8, 4096 - 5, 2048), (16, 2048 - 15, 512), (4, 1024 - 3, 256)])
+def test_padding_shorter_than_the_stride(S, L, C, use_triton):
+    """0 < padding < stride: the reshaped padding count is 0, so the torch branch's slice over "the last 0
+    reshaped keys" covers every key and each query chunk again sees only its own chunk
+    (xattn/src/Xattention.py:67,201); the Triton branch zeroes no row (kernels.py:70)."""
+    from xattn.src.Xattention import estimate_and_select
+
+    q, k = _mk(4, 2, L, L, 61, scale=1.5)
+    r = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=True, use_triton=use_triton)
+    want, want_mask = O.xattn_estimate(q.float(), k.repeat_interleave(2, 1).float(), 128, S, threshold=0.9,
+                                       chunk_size=C, causal=True, pad0_quirk=not use_triton)
+    assert torch.allclose(r["sums"].cpu(), want[0], rtol=2e-4, atol=2e-5), (r["sums"].cpu() - want[0]).abs().max()
+    nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, True, 0, C // 128)
+    assert outside == 0, (nbad, outside)

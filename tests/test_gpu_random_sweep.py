@@ -54,9 +54,10 @@ def test_random_configuration(c):
                                 **{**kw, "threshold": tau_dev})
     assert mask.shape == want_mask.shape
     assert torch.allclose(sums.float().cpu(), want_sums, rtol=1e-2, atol=2e-3)          # bf16 result of the operator
-    # (blocks the keep flags force are set on both sides and cannot mismatch)
+    # (blocks the keep flags force are set on both sides and cannot mismatch themselves)
     nq_p, nk_p = mask.shape[2], mask.shape[3]
-    nbad, outside = mask_mismatch_report(want_sums[0], mask[0], want_mask[0], tau, c["causal"], nk_p - nq_p, C // 128)
+    nbad, outside = mask_mismatch_report(want_sums[0], mask[0], want_mask[0], tau, c["causal"], nk_p - nq_p, C // 128,
+                                         keep_recent=c["keep_recent"])
     assert outside == 0, (nbad, outside)
 
     nq, nk = (Lq + 127) // 128, (Lk + 127) // 128

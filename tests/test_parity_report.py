@@ -127,3 +127,25 @@ def test_column_zero_comes_free_with_a_cut_run():
     got = want.clone()
     got[0, 7] = lowest
     assert mask_mismatch_detail(x[0], got, want, 0.5, True, 0, 32)["outside"] == 0
+
+
+def test_forced_diagonal_of_keep_recent_comes_free_without_causality():
+    """Non-causal row of six equal sums, tau 0.45: three are chosen (which three is the sort's business), then
+    keep_recent sets the diagonal (here column 4) and column 0 is set because ranks were left out.  A mask
+    whose picks include those columns shows fewer blocks than one whose picks avoid them."""
+    x = torch.ones(1, 1, 6)
+    picks_low = torch.tensor([[[True, True, True, False, True, False]]])      # picks 0,1,2; diagonal 4 forced
+    picks_mid = torch.tensor([[[True, True, True, True, True, False]]])       # picks 1,2,3; columns 0 and 4 come free
+    picks_hit = torch.tensor([[[True, True, False, False, True, False]]])     # picks 0,1,4: both free columns used up
+    for a in (picks_low, picks_mid, picks_hit):
+        for b in (picks_low, picks_mid, picks_hit):
+            d = mask_mismatch_detail(x, a, b, 0.45, False, 4, keep_recent=True)
+            assert d["outside"] == 0 and d["ties"] == d["mismatches"]
+    # without the flag the diagonal is an ordinary member of the run and the counts no longer agree
+    assert mask_mismatch_detail(x, picks_hit, picks_mid, 0.45, False, 4)["outside"] > 0
+    too_few = torch.tensor([[[True, False, False, False, True, False]]])      # only the free columns
+    assert mask_mismatch_detail(x, too_few, picks_mid, 0.45, False, 4, keep_recent=True)["outside"] > 0
+    # the oracle's own post-processed mask is one of the allowed outcomes
+    want = O.find_blocks_chunked(x[None], 0, 0.45, None, decoding=False, mode="prefill", causal=False)[0]
+    want[0, 0, 4] = True
+    assert mask_mismatch_detail(x, picks_low, want, 0.45, False, 4, keep_recent=True)["outside"] == 0

@@ -143,7 +143,9 @@ class _Plan:
         assert (self.k_len + k_pad) // chunk_size >= self.q_chunks
         self.nqb, self.nkb = (self.q_len + q_pad) // block_size, (self.k_len + k_pad) // block_size
         self.blocks_per_chunk = chunk_size // block_size
-        self.own_chunk_only = self.causal and (not use_triton) and k_pad == 0
+        # the torch branch hides "the last k_pad // stride reshaped keys" with a slice that covers every key
+        # when that count is 0 (xattn/src/Xattention.py:67,201) - also when 0 < k_pad < stride
+        self.own_chunk_only = self.causal and (not use_triton) and k_pad // stride == 0
         self.scale = 1.0 / math.sqrt(128) / stride / norm
         # Query rows (after subsampling) from which the block sums are all-zero.  Torch branch: the last
         # q_pad // stride // kdb rows of the last chunk - all of that chunk when that count is 0 but there is
