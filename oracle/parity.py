@@ -24,7 +24,9 @@ def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_c
     through, with both masks keeping as many of them as the rule allows: which members of
     such a run are kept is the order an unstable sort happens to give (the
     reference uses torch.sort, xattn/src/utils.py:110,126,150) or, for sums that
-    differ in the last bits, the order rounding gives;
+    differ in the last bits, the order rounding gives; when causal, the zero sums of
+    the blocks after the diagonal are members of a run of zeros too (the reference
+    sorts whole rows and clears those blocks afterwards), so a pick may vanish there;
     ``outside`` - everything else, i.e. real disagreements.  Forced blocks and
     blocks beyond the diagonal are never excused.  ``keep_recent`` says that the
     masks were post-processed with the block diagonal forced
@@ -54,16 +56,24 @@ def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_c
         if (h, i) not in rows:
             row = sums[h, i]
             total = float(row.sum())
-            limit = min(diag + 1, nk) if causal else nk
-            cols = np.array([c for c in range(limit) if c not in forced], dtype=np.int64)
+            # every column is a candidate of the reference's sort, blocks after the diagonal included: their
+            # sums are zero, so they only ever matter as members of a run of zeros (they are cleared afterwards)
+            cols = np.array([c for c in range(nk) if c not in forced], dtype=np.int64)
             vals = row[cols]
             order = np.lexsort((cols, -vals))          # descending sum, ascending column among equals
             vals, cols = vals[order], cols[order]
             base = float(sum(row[c] for c in forced if c < nk))
-            before = base + np.concatenate(([0.0], np.cumsum(vals)[:-1])) if len(vals) else np.zeros(0)
-            if one_forced and len(vals):
-                before = before - np.concatenate(([0.0], vals[:-1]))
-                before[0] = 0.0
+            csum = np.concatenate(([0.0], np.cumsum(vals)))             # csum[t] = the t largest ordinary sums
+            if causal:
+                # xattn/src/utils.py:107-141: the row is ranked by the sum for ordinary blocks and by
+                # 100000 * (1 + sum) for forced ones; rank r is judged against M(r), M(0) = M(1) = 0,
+                # M(r) = forced sum + the r - 2 largest ordinary sums.  The i-th ordinary block sits at rank
+                # i + (forced keys not below its own): i + 2 as a rule, i + 1 where only the diagonal is forced
+                fkeys = [100000.0 * (1.0 + row[c]) for c in forced if c < nk]
+                rank = np.arange(len(vals)) + np.array([sum(1 for f in fkeys if not v > f) for v in vals], dtype=np.int64)
+                before = np.where(rank < 2, 0.0, base + csum[np.maximum(rank - 2, 0)])
+            else:
+                before = csum[:-1]
             need = taus[h].item() * total
             near = np.abs(before - need) <= TAU_BAND * max(total, 1e-30)
             rows[(h, i)] = (row, vals, cols, near, before < need)
@@ -79,8 +89,10 @@ def mask_mismatch_detail(sums, got, want, tau, causal, diag_offset, blocks_per_c
             # anyway (unselected ranks scatter to it), and so is the diagonal under keep_recent: a mask may
             # show one chosen member fewer beside each such member
             free = [c for c in ([0, diag] if keep_recent and not causal else [0]) if c in run]
-            rest = run[~np.isin(run, free)]
-            counts = set(range(kept - len(free), kept + 1))
+            visible = run[run <= diag] if causal else run
+            rest = visible[~np.isin(visible, free)]
+            # picks that land on members after the diagonal are cleared again and show nowhere
+            counts = set(range(max(0, kept - len(free) - (len(run) - len(visible))), kept + 1))
             ok = all(int(m[h, i][rest].sum()) in counts and all(bool(m[h, i][c]) for c in free) for m in (got, want))
             if ok:
                 ties += 1

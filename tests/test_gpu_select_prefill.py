@@ -189,3 +189,28 @@ def test_operator_with_kv_longer_than_q():
     if nbad == 0:
         err = (out.float().cpu() - want.float()).abs()
         assert err.max().item() <= OUT_MAX_ABS and err.mean().item() <= OUT_MEAN_ABS
+
+
+def test_sums_beyond_a_forced_key_move_up_in_rank():
+    """Un-normalised block sums (softmax=False) above 100000 * (1 + forced sum) rank before that forced block
+    in the reference (xattn/src/utils.py:126-130) and are judged against less mass; hand-worked rows (see the
+    oracle's test of the same name) and random rows whose sums straddle the forced keys."""
+    rows = [([10.0, 5e6, 3e6, 2.0, 50.0], 4, 0.5, [1, 1, 1, 0, 1, 0, 0, 0]),
+            ([10.0, 90.0, 30.0, 2.0, 50.0], 4, 0.5, [1, 1, 0, 0, 1, 0, 0, 0]),
+            ([1.0, 4e5, 3.5e5, 1e5, 9e4, 2.0], 5, 0.85, [1, 1, 1, 1, 0, 1, 0, 0])]
+    for vals, diag, tau, want in rows:
+        x = torch.zeros(1, 1, 8)
+        x[0, 0, : len(vals)] = torch.tensor(vals)
+        got, _, _ = _select(x, tau, True, diag)
+        assert got[0, 0].int().tolist() == want, (vals, got[0, 0].int().tolist())
+    g = torch.Generator().manual_seed(11)
+    for nk, off in [(40, 8), (300, 268), (1500, 1468), (32, 0)]:           # extraction path, sort path, first chunk
+        nq = 32
+        x = torch.exp(torch.rand(4, nq, nk, generator=g) * 18.0)             # sums from 1 to 6e7
+        vis = torch.arange(nk)[None, :] <= torch.arange(nq)[:, None] + off
+        x = x * vis
+        taus = torch.tensor([0.3, 0.6, 0.9, 0.99])
+        got, _, _ = _select(x, taus, True, off)
+        want = O.find_blocks_chunked(x[None], off, taus, None, decoding=False, mode="prefill", causal=True)[0] & vis
+        nbad, outside = mask_mismatch_report(x, got, want, taus, True, off)
+        assert outside == 0, (nk, off, nbad, outside)

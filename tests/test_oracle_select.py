@@ -166,3 +166,28 @@ def test_decode_mode_of_find_blocks_chunked():
         with pytest.raises(RuntimeError):
             f(x, 0, 0.9, None, decoding=False, mode="decode", causal=True)         # 1 row against 3
         assert f(x, 0, 0.9, None, decoding=True, mode="prefill").all()
+
+
+def test_sums_beyond_a_forced_key_move_up_in_rank():
+    """Hand-worked: the reference ranks forced blocks by 100000 * (1 + sum) and the rest by their sum
+    (xattn/src/utils.py:126-130); rank r is kept while M(r) < tau * total with M = cumsum([0, 0, forced_sum,
+    others...]) (:115-141).  Un-normalised sums (softmax=False) can exceed a forced key.  Row with sink 10,
+    diagonal 50 (keys 1.1e6 and 5.1e6) and others 5e6, 3e6, 2: order [diag, 5e6, 3e6, sink, 2], masses
+    [0, 0, 60, 60 + 5e6, ...] against 0.5 * 8000062: both big blocks are kept - with the forced blocks ranked
+    first the second one (mass 60 + 5e6) would not be."""
+    x = torch.zeros(1, 1, 1, 8, dtype=torch.float32)
+    x[0, 0, 0, :5] = torch.tensor([10.0, 5e6, 3e6, 2.0, 50.0])
+    want = O.find_blocks_chunked(x, 4, 0.5, None, decoding=False, mode="prefill", causal=True)[0, 0, 0]
+    assert want.tolist() == [True, True, True, False, True, False, False, False]
+    # below 100000 nothing changes rank: sink 10, diagonal 50, others 90, 30, 2 (total 182, need 91): the first
+    # other is judged against 60, the second against 150
+    y = torch.zeros(1, 1, 1, 8, dtype=torch.float32)
+    y[0, 0, 0, :5] = torch.tensor([10.0, 90.0, 30.0, 2.0, 50.0])
+    got = O.find_blocks_chunked(y, 4, 0.5, None, decoding=False, mode="prefill", causal=True)[0, 0, 0]
+    assert got.tolist() == [True, True, False, False, True, False, False, False]
+    # a sum beyond BOTH keys takes rank 0: sink 1, diagonal 2 (keys 2e5, 3e5), others 4e5, 3.5e5, 1e5, 9e4
+    # order [4e5, 3.5e5, diag, sink, 1e5, 9e4]; masses [0, 0, 3, 3 + 4e5, 3 + 7.5e5, ...]; need 0.85 * 940003
+    z = torch.zeros(1, 1, 1, 8, dtype=torch.float32)
+    z[0, 0, 0, :6] = torch.tensor([1.0, 4e5, 3.5e5, 1e5, 9e4, 2.0])
+    got = O.find_blocks_chunked(z, 5, 0.85, None, decoding=False, mode="prefill", causal=True)[0, 0, 0]
+    assert got.tolist() == [True, True, True, True, False, True, False, False]

@@ -149,3 +149,33 @@ def test_forced_diagonal_of_keep_recent_comes_free_without_causality():
     want = O.find_blocks_chunked(x[None], 0, 0.45, None, decoding=False, mode="prefill", causal=False)[0]
     want[0, 0, 4] = True
     assert mask_mismatch_detail(x, picks_low, want, 0.45, False, 4, keep_recent=True)["outside"] == 0
+
+
+def test_a_pick_among_zero_sums_may_land_after_the_diagonal():
+    """First query chunk, row 2 of a 6-column grid, sums [a, 0, 0 | 0, 0, 0]: the rule keeps the diagonal, column 0
+    and ONE of the zero-sum blocks; the reference sorts all six columns, so that pick is column 1 or one of the
+    three blocks after the diagonal, which are cleared afterwards.  Both outcomes are the reference's."""
+    x = torch.zeros(1, 3, 6)
+    x[0, 0, 0] = 1.0
+    x[0, 1, :2] = torch.tensor([0.5, 0.5])
+    x[0, 2, 0] = 0.0645
+    a = torch.zeros(1, 3, 6, dtype=torch.bool)
+    a[0, 0, 0] = a[0, 1, 0] = a[0, 1, 1] = True
+    b = a.clone()
+    a[0, 2, :3] = torch.tensor([True, True, True])       # the pick landed on column 1
+    b[0, 2, :3] = torch.tensor([True, False, True])      # ... or after the diagonal
+    d = mask_mismatch_detail(x, a, b, 0.5, True, 0, 3)
+    assert d == {"mismatches": 1, "in_band": 0, "ties": 1, "outside": 0}
+    # the oracle's own answer is one of the two
+    want = O.find_blocks_chunked(x[None], 0, 0.5, None, decoding=False, mode="prefill", causal=True)[0]
+    want &= torch.arange(6)[None, :] <= torch.arange(3)[:, None]
+    assert mask_mismatch_detail(x, a, want, 0.5, True, 0, 3)["outside"] == 0
+    assert mask_mismatch_detail(x, b, want, 0.5, True, 0, 3)["outside"] == 0
+    # keeping BOTH zero-sum candidates of a longer row is one pick too many
+    x2 = torch.zeros(1, 4, 6)
+    x2[0, 3, 0] = 0.0645
+    w2 = torch.zeros(1, 4, 6, dtype=torch.bool)
+    w2[0, 3, [0, 1, 3]] = True
+    g2 = w2.clone()
+    g2[0, 3, 2] = True
+    assert mask_mismatch_detail(x2, g2, w2, 0.5, True, 0, 4)["outside"] == 1

@@ -14,6 +14,18 @@
 // ascending column among equals) and apply the same rule.  The kernel emits the
 // final mask row plus the compacted, ascending column list the attention kernel
 // walks.
+//
+// The causal rule, as the reference's tensors define it (utils.py:107-141): the
+// row is ranked by a key that is the block sum for ordinary blocks and
+// 100000 * (1 + sum) for the forced ones; rank r is kept while M(r) < tau *
+// total, with M(0) = M(1) = 0 and M(r) = forced_sum + the r - 2 largest
+// ordinary sums.  With softmax block sums (at most block_size / stride per
+// block) the forced blocks always rank first, so the i-th largest ordinary
+// block sits at rank i + 2 (i + 1 in the first query chunk, where only the
+// diagonal is forced) - but un-normalised sums (softmax = 0) can exceed a
+// forced key, and such a block then moves up one or two ranks.  rank_mass()
+// implements exactly that: the i-th ordinary block with `ahead` forced keys
+// before it is judged against M(i + ahead).
 #include "xattn_common.h"
 #include "xattn_hip.h"
 
@@ -46,6 +58,14 @@ __device__ __forceinline__ double wave_sum(double x) {
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) x += __shfl_xor(x, d, 64);
   return x;
+}
+
+// M(i + ahead) from the masses before the i-th ordinary block (b0), before its predecessor (b1) and before
+// the one ahead of that (b2); ranks 0 and 1 carry no mass
+__device__ __forceinline__ double rank_mass(int i, int ahead, double b0, double b1, double b2) {
+  const int back = 2 - ahead;          // 0, 1 or 2 ordinary blocks fewer than all those ahead of it
+  if (i < back) return 0.0;
+  return back == 0 ? b0 : (back == 1 ? b1 : b2);
 }
 
 __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
@@ -112,10 +132,22 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   total = wave_sum(total);
   const double required = total * p.tau[head];
   double forced_sum = 0.0;
+  // sort keys of the forced blocks (utils.py:126-130); key_hi >= key_lo, equal when only one block is forced
+  double key_lo = 0.0, key_hi = 0.0;
   if (p.causal && ncand > 0) {
     if (!one_forced || diag == 0) forced_sum = (double)x[0];
     if (diag != 0 && diag < p.nkb) forced_sum += (double)x[diag];
+    const double kd = 100000.0 * (1.0 + (double)x[diag < p.nkb ? diag : 0]);
+    const double k0 = one_forced ? kd : 100000.0 * (1.0 + (double)x[0]);
+    key_lo = kd < k0 ? kd : k0;
+    key_hi = kd < k0 ? k0 : kd;
   }
+  const int n_forced = one_forced ? 1 : 2;
+  // forced keys ranked ahead of an ordinary block of sum v (all of them unless v is beyond 100000)
+  auto forced_ahead = [&](double v) -> int {
+    if (!(v > key_lo)) return n_forced;
+    return one_forced ? 0 : (v > key_hi ? 0 : 1);
+  };
   __syncthreads();
 
   int dropped = 0;
@@ -124,12 +156,10 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     // ---- extraction: keep pulling out the largest remaining block while the rule says "keep"
 #pragma unroll
     for (int d = 32; d > 0; d >>= 1) n_others += __shfl_xor(n_others, d, 64);
-    double before = forced_sum, prev_before = 0.0;
+    double before = forced_sum, prev_before = 0.0, prev2_before = 0.0;
     for (int it = 0; it < kMaxExtract; ++it) {
-      const double mass = one_forced ? (it == 0 ? 0.0 : prev_before) : before;
-      if (!(mass < required) || n_others == 0) {
+      if (n_others == 0) {
         finished = true;
-        dropped = n_others > 0;
         break;
       }
       uint32_t best = 0;
@@ -139,6 +169,13 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
       for (int d = 32; d > 0; d >>= 1) {
         const uint32_t o = __shfl_xor(best, d, 64);
         best = o > best ? o : best;
+      }
+      const double best_val = (double)__uint_as_float(best - 1u);
+      const double mass = p.causal ? rank_mass(it, forced_ahead(best_val), before, prev_before, prev2_before) : before;
+      if (!(mass < required)) {
+        finished = true;
+        dropped = 1;
+        break;
       }
       uint32_t col = 0xffffffffu;     // lowest column holding the maximum
 #pragma unroll
@@ -151,8 +188,9 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
 #pragma unroll
       for (int u = 0; u < kSlots; ++u) vals[u] = (uint32_t)(u * 64 + lane) == col ? 0u : vals[u];
       if (lane == 0) flags[col] = 1;
+      prev2_before = prev_before;
       prev_before = before;
-      before += (double)__uint_as_float(best - 1u);
+      before += best_val;
       --n_others;
     }
   }
@@ -192,7 +230,11 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     const uint32_t col = ~(uint32_t)key;
     if (col < (uint32_t)ncand && (key >> 32) != 0) {
       double mass = before;
-      if (one_forced) mass = rank == 0 ? 0.0 : before - key_value(keys[rank - 1]);
+      if (p.causal) {
+        const double b1 = rank > 0 ? before - key_value(keys[rank - 1]) : 0.0;
+        const double b2 = rank > 1 ? b1 - key_value(keys[rank - 2]) : 0.0;
+        mass = rank_mass(rank, forced_ahead(key_value(key)), before, b1, b2);
+      }
       if (mass < required) flags[col] = 1;
       else dropped = 1;
     }
