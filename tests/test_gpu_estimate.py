@@ -260,3 +260,23 @@ def test_padding_shorter_than_the_stride(S, L, C, use_triton):
     assert torch.allclose(r["sums"].cpu(), want[0], rtol=2e-4, atol=2e-5), (r["sums"].cpu() - want[0]).abs().max()
     nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, True, 0, C // 128)
     assert outside == 0, (nbad, outside)
+
+
+@pytest.mark.parametrize("causal,use_triton", [(True, True), (True, False), (False, True)])
+def test_more_tiles_than_compute_units(causal, use_triton):
+    """S=4 at 12k tokens and 8 heads is 600-1200 tiles of 256x256: every workgroup of the estimator then works
+    through several tiles (the next tile's first slabs are requested before the current tile's epilogue), with
+    a ragged last tile and a cached prefix."""
+    from xattn.src.Xattention import estimate_and_select
+
+    S, C, Lq, Lk = 4, 2048, 12288 - 37, 12288 + 1024 - 37
+    if not causal:
+        Lk = Lq
+    q, k = _mk(8, 2, Lq, Lk, 77, scale=1.5)
+    r = estimate_and_select(q.cuda(), k.cuda(), S, 0.9, C, causal=causal, use_triton=use_triton)
+    want, want_mask = O.xattn_estimate(q.float(), k.repeat_interleave(4, 1).float(), 128, S, threshold=0.9,
+                                       chunk_size=C, causal=causal, pad0_quirk=not use_triton)
+    assert torch.allclose(r["sums"].cpu(), want[0], rtol=2e-4, atol=2e-5), (r["sums"].cpu() - want[0]).abs().max()
+    nq_p, nk_p = want_mask.shape[2], want_mask.shape[3]
+    nbad, outside = mask_mismatch_report(want[0], r["mask"], want_mask[0], 0.9, causal, nk_p - nq_p, C // 128)
+    assert outside == 0, (nbad, outside)

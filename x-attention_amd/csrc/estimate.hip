@@ -18,6 +18,8 @@
 //  kernel 2 (estimate_normalize_kernel): per query row, combines the tile
 //    maxima/sums into the row's softmax statistics, rescales the partial sums
 //    and adds the block_size/S rows of each query block.
+#include <mutex>
+
 #include "xattn_common.h"
 #include "xattn_hip.h"
 
@@ -108,6 +110,40 @@ __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk
 }
 
 
+// Tile assignment.  Only tiles holding a visible (row, key) pair are
+// enumerated: per KV group, by query tile row, then key tile, then query head
+// of the group.  Tile ids are dealt round-robin to the 8 XCDs (workgroup b
+// runs on XCD b % 8 and takes ids b, b + grid, ... with the grid a multiple of
+// 8), so runs of 32 consecutive tiles are given to one XCD: the 32 tiles an XCD
+// works on at a time are then 8 key tiles x the heads of one group for one
+// query tile row, which share their K' slabs across heads and their Q' slabs
+// across key tiles in that XCD's L2, and every XCD gets the same number of tiles.
+// Returns false when id is past the last tile.
+__device__ __forceinline__ bool decode_tile(const EstParams& p, int64_t id, int* head, int* m0, int* n0) {
+  const int64_t lin = ((id >> 8) * 8 + (id & 7)) * 32 + ((id >> 3) & 31);
+  if (lin >= p.total_tiles) return false;
+  const int G = p.H / p.Hkv;
+  const int per_group = p.tiles_per_head * G;
+  const int g = (int)(lin / per_group);
+  int rem = (int)(lin % per_group);
+  *head = g * G + rem % G;
+  int tt = rem / G;
+  int mt_row = 0, nt_first = 0;
+  for (;; ++mt_row) {
+    const int mfirst = p.row_begin + mt_row * kTile;
+    const int mlast = (mfirst + kTile - 1 < p.row_end ? mfirst + kTile - 1 : p.row_end - 1);
+    int hi = row_hi(p, mlast) / kTile;
+    hi = hi < p.nNT - 1 ? hi : p.nNT - 1;
+    nt_first = row_lo(p, mfirst) / kTile;
+    const int cnt = hi - nt_first + 1;
+    if (tt < cnt || mt_row + 1 >= p.nMT) break;
+    tt -= cnt;
+  }
+  *m0 = p.row_begin + mt_row * kTile;
+  *n0 = (nt_first + tt) * kTile;
+  return true;
+}
+
 // kDump: also write the raw scores (test / seam builds only; kept out of the production instantiation)
 // kTable: the depth slabs come from p.pairs (the non-default select modes); the default keeps its closed form
 template <int RBS, bool kDump, bool kTable>
@@ -118,70 +154,31 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, hh = lane >> 5;
   const int wm = wave & 3, wn = wave >> 2;   // query quarter, key half
-  // Tile assignment.  Only tiles holding a visible (row, key) pair are
-  // enumerated: per KV group, by query tile row, then key tile, then query head
-  // of the group.  Workgroup ids are dealt round-robin to the 8 XCDs, so runs of
-  // 32 consecutive tiles are given to one XCD: the 32 tiles an XCD works on at a
-  // time are then 8 key tiles x the heads of one group for one query tile row,
-  // which share their K' slabs across heads and their Q' slabs across key tiles
-  // in that XCD's L2, and every XCD gets the same number of tiles.
+  // A workgroup works through tiles id, id + grid, ...: one workgroup fits a CU, so nothing else could hide
+  // the wait for a tile's first slabs - instead the first slabs of the NEXT tile are requested before the
+  // epilogue of the current one (which needs no LDS) and land while it runs.
+  int64_t id = blockIdx.x;
   int head, m0, n0;
-  {
-    const int id = blockIdx.x;
-    const int64_t lin = ((int64_t)(id >> 8) * 8 + (id & 7)) * 32 + ((id >> 3) & 31);
-    if (lin >= p.total_tiles) return;
-    const int G = p.H / p.Hkv;
-    const int per_group = p.tiles_per_head * G;
-    const int g = (int)(lin / per_group);
-    int rem = (int)(lin % per_group);
-    head = g * G + rem % G;
-    int tt = rem / G;
-    int mt_row = 0, nt_first = 0;
-    for (;; ++mt_row) {
-      const int mfirst = p.row_begin + mt_row * kTile;
-      const int mlast = (mfirst + kTile - 1 < p.row_end ? mfirst + kTile - 1 : p.row_end - 1);
-      int hi = row_hi(p, mlast) / kTile;
-      hi = hi < p.nNT - 1 ? hi : p.nNT - 1;
-      nt_first = row_lo(p, mfirst) / kTile;
-      const int cnt = hi - nt_first + 1;
-      if (tt < cnt || mt_row + 1 >= p.nMT) break;
-      tt -= cnt;
-    }
-    m0 = p.row_begin + mt_row * kTile;
-    n0 = (nt_first + tt) * kTile;
-  }
+  if (!decode_tile(p, id, &head, &m0, &n0)) return;
 
-  // (kept as a guard) tiles without a visible (row, key) pair do nothing
-  {
-    const int m_last = (m0 + kTile - 1 < p.row_end ? m0 + kTile - 1 : p.row_end - 1);
-    if (n0 > row_hi(p, m_last)) return;
-    if (n0 + kTile - 1 < row_lo(p, m0)) return;
-  }
-
-  const int kvh = head / (p.H / p.Hkv);
-  const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
-  const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
+  const int64_t q_snb = p.q_sn * 2, k_snb = p.k_sn * 2;
+  const int64_t span = (int64_t)kTile * p.S;
   // Buffer resources are rebased to the tile's first token and end at the real
   // sequence end (or the tile's end), so lane offsets stay small whatever the
   // token stride, and tokens past the real length read as zeros.
-  const int64_t q_snb = p.q_sn * 2, k_snb = p.k_sn * 2;
-  const int64_t q_tok0 = (int64_t)m0 * p.S * p.kdb, k_tok0 = (int64_t)n0 * p.S;
-  const int64_t q_left = p.Lq - q_tok0, k_left = p.Lk - k_tok0;
-  const int64_t span = (int64_t)kTile * p.S;
-  const int64_t q_rows = q_left < 0 ? 0 : (q_left < span * p.kdb ? q_left : span * p.kdb);
-  const int64_t k_rows = k_left < 0 ? 0 : (k_left < span ? k_left : span);
-  const __amdgpu_buffer_rsrc_t qres = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(qbase + (q_rows > 0 ? q_tok0 * p.q_sn : 0)), 0, (int)(q_rows * q_snb), 0x00020000);
-  const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)(kbase + (k_rows > 0 ? k_tok0 * p.k_sn : 0)), 0, (int)(k_rows * k_snb), 0x00020000);
-
-  f32x16 acc[4][2];   // [key tile nt][query tile mt]
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+  auto q_resource = [&](int h, int m) {
+    const int64_t tok0 = (int64_t)m * p.S * p.kdb, left = p.Lq - tok0;
+    const int64_t rows = left < 0 ? 0 : (left < span * p.kdb ? left : span * p.kdb);
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(p.q + (int64_t)h * p.q_sh + (rows > 0 ? tok0 * p.q_sn : 0)), 0,
+                                             (int)(rows * q_snb), 0x00020000);
+  };
+  auto k_resource = [&](int h, int n) {
+    const int64_t tok0 = (int64_t)n * p.S, left = p.Lk - tok0;
+    const int64_t rows = left < 0 ? 0 : (left < span ? left : span);
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(p.k + (int64_t)(h / (p.H / p.Hkv)) * p.k_sh + (rows > 0 ? tok0 * p.k_sn : 0)),
+                                             0, (int)(rows * k_snb), 0x00020000);
+  };
+  __amdgpu_buffer_rsrc_t qres = q_resource(head, m0), kres = k_resource(head, n0);
 
   // k-step t covers token i = t / 2 of every reshaped row's group, features
   // 64*(t % 2) .. +63, and is read from LDS stage t % 2.
@@ -208,17 +205,30 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     return i * (int)q_snb + (t & 1) * kDepth * 2;
   };
   // copy j (0..7) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
-  auto copy_j = [&](int j, int t, char* stage) {
+  auto copy_j = [&](__amdgpu_buffer_rsrc_t qr, __amdgpu_buffer_rsrc_t kr, int j, int t, char* stage) {
     const int tc = t < steps ? t : steps - 1;       // past the end: a harmless repeat
-    if (j & 1) copy_one(qres, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
-    else copy_one(kres, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
+    if (j & 1) copy_one(qr, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
+    else copy_one(kr, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
   };
+  // a tile's first requests: all of step 0 and the first two copies of step 1
+  auto first_copies = [&](__amdgpu_buffer_rsrc_t qr, __amdgpu_buffer_rsrc_t kr) {
 #pragma unroll
-  for (int j = 0; j < 8; ++j) copy_j(j, 0, lds);
+    for (int j = 0; j < 8; ++j) copy_j(qr, kr, j, 0, lds);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) copy_j(qr, kr, j, 1, lds + kStageBytes);
+  };
+  first_copies(qres, kres);
+
+  for (;;) {
+  f32x16 acc[4][2];   // [key tile nt][query tile mt]
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
   wait_vm0();
-  __syncthreads();
-#pragma unroll
-  for (int j = 0; j < 2; ++j) copy_j(j, 1, lds + kStageBytes);
+  __syncthreads();        // this tile's first slabs have landed and are visible
 
   bf16x8 fa[2][4], fb[2][2];
 #pragma unroll
@@ -245,8 +255,8 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
       for (int c = 0; c < 4; ++c) {
         __builtin_amdgcn_sched_barrier(0);
         if (c < 2) {
-          if (ss < 3) copy_j(2 + ss * 2 + c, t + 1, nxt);  // copies 2..7 of step t+1
-          else copy_j(c, t + 2, cur);                      // copies 0..1 of step t+2 refill this stage
+          if (ss < 3) copy_j(qres, kres, 2 + ss * 2 + c, t + 1, nxt);  // copies 2..7 of step t+1
+          else copy_j(qres, kres, c, t + 2, cur);                      // copies 0..1 of step t+2 refill this stage
           fa[(ss + 1) & 1][2 * c] = read_frag(fragK, wn * kSub + (2 * c) * 32 + r, nss * 2 + hh);
           fa[(ss + 1) & 1][2 * c + 1] = read_frag(fragK, wn * kSub + (2 * c + 1) * 32 + r, nss * 2 + hh);
         } else if (c == 2) {
@@ -261,10 +271,22 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   }
   wait_vm0();   // the repeats issued by the last steps
 
+  // Every fragment of this tile has been read (the last barrier sits before the last sub-step), so the stages
+  // are free: the next tile's first slabs are requested now and arrive during the epilogue.
+  const int64_t id_next = id + gridDim.x;
+  int head_next, m0_next, n0_next;
+  const bool more = decode_tile(p, id_next, &head_next, &m0_next, &n0_next);
+  __amdgpu_buffer_rsrc_t qres_next = qres, kres_next = kres;
+  if (more) {
+    qres_next = q_resource(head_next, m0_next);
+    kres_next = k_resource(head_next, n0_next);
+    first_copies(qres_next, kres_next);
+  }
+
   // ---- epilogue: this wavefront's 128 keys x 64 query rows
   const int nbase = n0 + wn * kSub;       // first key of the wavefront tile
   const int T = nbase / kSub;
-  if (nbase >= p.n_rk) return;
+  if (nbase < p.n_rk) {
   float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
   float* Mst = p.Mt + ((int64_t)head * p.nT + T) * p.rows;
   float* Lst = p.Lt + ((int64_t)head * p.nT + T) * p.rows;
@@ -356,6 +378,16 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     // keep the query-tile passes apart: interleaving them only lengthens live ranges
     __builtin_amdgcn_sched_barrier(0);
   }
+  }   // epilogue
+
+  if (!more) break;
+  id = id_next;
+  head = head_next;
+  m0 = m0_next;
+  n0 = n0_next;
+  qres = qres_next;
+  kres = kres_next;
+  }   // tiles of this workgroup
 }
 
 // One workgroup = 64 consecutive reshaped query rows of one head.
@@ -536,6 +568,21 @@ hipError_t launch_gemm(const EstParams& p, dim3 grid, size_t lds, hipStream_t s)
   return hipSuccess;
 }
 
+// CUs of the current device, rounded down to a multiple of 8 (tile ids are dealt to the 8 XCDs in turn)
+int resident_workgroups() {
+  static std::mutex mu;
+  static int per_device[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  std::lock_guard<std::mutex> lock(mu);
+  if (per_device[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    per_device[dev] = cus >= 8 ? cus / 8 * 8 : 8;
+  }
+  return per_device[dev];
+}
+
 struct Geometry {
   int q_pad, k_pad, n_rq, n_rk, nqb, nkb, nT, rcs, q_chunks;   // n_rq: reshaped query rows before subsampling
 };
@@ -658,7 +705,10 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   p.total_tiles = (int64_t)p.tiles_per_head * num_heads;
   const int64_t ids = (p.total_tiles + 255) / 256 * 256;
   if (ids > 0x7fffffff) return XATTN_ERR_SHAPE;
-  const dim3 grid1((unsigned)ids);
+  // one workgroup per CU (its LDS stages fill a CU), each working through tile ids b, b + grid, ...
+  const int resident = resident_workgroups();
+  if (resident <= 0) return XATTN_ERR_LAUNCH;
+  const dim3 grid1((unsigned)(ids < resident ? ids : resident));
   const dim3 grid2((p.rows + 63) / 64, num_heads);
   if (grid2.y > 65535) return XATTN_ERR_SHAPE;
   const size_t lds = 2 * (size_t)kStageBytes;
