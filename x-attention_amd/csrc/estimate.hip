@@ -155,8 +155,9 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   const int r = lane & 31, hh = lane >> 5;
   const int wm = wave & 3, wn = wave >> 2;   // query quarter, key half
   // A workgroup works through tiles id, id + grid, ...: one workgroup fits a CU, so nothing else could hide
-  // the wait for a tile's first slabs - instead the first slabs of the NEXT tile are requested before the
-  // epilogue of the current one (which needs no LDS) and land while it runs.
+  // the wait for a tile's first slabs.  The copy pipeline therefore runs on across the tile boundary: the copy
+  // slots of a tile's last two k-steps fetch the first slabs of the NEXT tile, and the last sub-step reads its
+  // first fragments, so after the epilogue (which needs no LDS) the next tile starts at full speed.
   int64_t id = blockIdx.x;
   int head, m0, n0;
   if (!decode_tile(p, id, &head, &m0, &n0)) return;
@@ -179,6 +180,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
                                              0, (int)(rows * k_snb), 0x00020000);
   };
   __amdgpu_buffer_rsrc_t qres = q_resource(head, m0), kres = k_resource(head, n0);
+  __amdgpu_buffer_rsrc_t qres_next = qres, kres_next = kres;
 
   // k-step t covers token i = t / 2 of every reshaped row's group, features
   // 64*(t % 2) .. +63, and is read from LDS stage t % 2.
@@ -204,22 +206,36 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     const int i = kTable ? (p.pairs[t >> 1] >> 4) : (p.S - 1 - (t >> 1));
     return i * (int)q_snb + (t & 1) * kDepth * 2;
   };
-  // copy j (0..7) of a step: slab rows it = j / 2 of K' (j even) or Q' (j odd)
-  auto copy_j = [&](__amdgpu_buffer_rsrc_t qr, __amdgpu_buffer_rsrc_t kr, int j, int t, char* stage) {
-    const int tc = t < steps ? t : steps - 1;       // past the end: a harmless repeat
-    if (j & 1) copy_one(qr, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
-    else copy_one(kr, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
+  // copy j (0..7) of k-step t: slab rows it = j / 2 of K' (j even) or Q' (j odd).  Steps `steps` and
+  // `steps + 1` are steps 0 and 1 of the next tile (of this tile again when it is the workgroup's last:
+  // a harmless repeat nobody reads).
+  auto copy_j = [&](int j, int t, char* stage) {
+    const bool ahead = t >= steps;
+    const int tc = ahead ? t - steps : t;
+    if (j & 1) copy_one(ahead ? qres_next : qres, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
+    else copy_one(ahead ? kres_next : kres, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
   };
-  // a tile's first requests: all of step 0 and the first two copies of step 1
-  auto first_copies = [&](__amdgpu_buffer_rsrc_t qr, __amdgpu_buffer_rsrc_t kr) {
+  // the workgroup's first tile: all of step 0 and the first two copies of step 1, then its first fragments
 #pragma unroll
-    for (int j = 0; j < 8; ++j) copy_j(qr, kr, j, 0, lds);
+  for (int j = 0; j < 8; ++j) copy_j(j, 0, lds);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) copy_j(qr, kr, j, 1, lds + kStageBytes);
-  };
-  first_copies(qres, kres);
+  for (int j = 0; j < 2; ++j) copy_j(j, 1, lds + kStageBytes);
+  wait_vm0();
+  __syncthreads();
+  bf16x8 fa[2][4], fb[2][2];
+#pragma unroll
+  for (int x = 0; x < 4; ++x) fa[0][x] = read_frag(lds, wn * kSub + x * 32 + r, hh);
+#pragma unroll
+  for (int x = 0; x < 2; ++x) fb[0][x] = read_frag(lds + kTile * 128, wm * kRowsW + x * 32 + r, hh);
 
   for (;;) {
+  const int64_t id_next = id + gridDim.x;
+  int head_next, m0_next, n0_next;
+  const bool more = decode_tile(p, id_next, &head_next, &m0_next, &n0_next);
+  if (more) {
+    qres_next = q_resource(head_next, m0_next);
+    kres_next = k_resource(head_next, n0_next);
+  }
   f32x16 acc[4][2];   // [key tile nt][query tile mt]
 #pragma unroll
   for (int a = 0; a < 4; ++a)
@@ -227,14 +243,6 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
-  wait_vm0();
-  __syncthreads();        // this tile's first slabs have landed and are visible
-
-  bf16x8 fa[2][4], fb[2][2];
-#pragma unroll
-  for (int x = 0; x < 4; ++x) fa[0][x] = read_frag(lds, wn * kSub + x * 32 + r, hh);
-#pragma unroll
-  for (int x = 0; x < 2; ++x) fb[0][x] = read_frag(lds + kTile * 128, wm * kRowsW + x * 32 + r, hh);
 
   for (int t = 0; t < steps; ++t) {
     char* cur = lds + (t & 1) * kStageBytes;
@@ -255,8 +263,8 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
       for (int c = 0; c < 4; ++c) {
         __builtin_amdgcn_sched_barrier(0);
         if (c < 2) {
-          if (ss < 3) copy_j(qres, kres, 2 + ss * 2 + c, t + 1, nxt);  // copies 2..7 of step t+1
-          else copy_j(qres, kres, c, t + 2, cur);                      // copies 0..1 of step t+2 refill this stage
+          if (ss < 3) copy_j(2 + ss * 2 + c, t + 1, nxt);  // copies 2..7 of step t+1
+          else copy_j(c, t + 2, cur);                      // copies 0..1 of step t+2 refill this stage
           fa[(ss + 1) & 1][2 * c] = read_frag(fragK, wn * kSub + (2 * c) * 32 + r, nss * 2 + hh);
           fa[(ss + 1) & 1][2 * c + 1] = read_frag(fragK, wn * kSub + (2 * c + 1) * 32 + r, nss * 2 + hh);
         } else if (c == 2) {
@@ -269,19 +277,8 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  wait_vm0();   // the repeats issued by the last steps
-
-  // Every fragment of this tile has been read (the last barrier sits before the last sub-step), so the stages
-  // are free: the next tile's first slabs are requested now and arrive during the epilogue.
-  const int64_t id_next = id + gridDim.x;
-  int head_next, m0_next, n0_next;
-  const bool more = decode_tile(p, id_next, &head_next, &m0_next, &n0_next);
-  __amdgpu_buffer_rsrc_t qres_next = qres, kres_next = kres;
-  if (more) {
-    qres_next = q_resource(head_next, m0_next);
-    kres_next = k_resource(head_next, n0_next);
-    first_copies(qres_next, kres_next);
-  }
+  // fa[0] / fb[0] now hold the first fragments of the next tile, whose step 0 sits in stage 0 and whose step 1
+  // is on its way into stage 1
 
   // ---- epilogue: this wavefront's 128 keys x 64 query rows
   const int nbase = n0 + wn * kSub;       // first key of the wavefront tile
@@ -388,6 +385,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   qres = qres_next;
   kres = kres_next;
   }   // tiles of this workgroup
+  wait_vm0();   // the repeats the last tile issued into LDS
 }
 
 // One workgroup = 64 consecutive reshaped query rows of one head.

@@ -101,32 +101,34 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   int n_others = 0;
 #pragma unroll
   for (int u = 0; u < kSlots; ++u) vals[u] = 0;
-  auto load_one = [&](int c) -> uint32_t {
-    uint64_t key = 0;   // padding sorts last and carries an out-of-range column
+  // value bits of candidate c (0 for forced blocks and columns past the candidates); adds it to `total` on request
+  auto load_one = [&](int c, bool count) -> uint32_t {
     uint32_t bits = 0;
     if (c < ncand) {
       const float v = x[c];
-      total += (double)v;
+      if (count) total += (double)v;
       const bool forced = p.causal && (c == diag || (c == 0 && !one_forced));
       // block sums are >= 0, so their bit pattern orders like the value (+1
-      // keeps every candidate ahead of the forced blocks, which sort last);
-      // low word = ~column makes equal sums come out by ascending column
+      // keeps every candidate ahead of the forced blocks, which sort last)
       bits = forced ? 0u : __float_as_uint(v > 0.f ? v : 0.f) + 1u;
-      key = ((uint64_t)bits << 32) | (uint32_t)(~(uint32_t)c);
     }
-    keys[c] = key;
     return bits;
   };
+  // sort key: low word = ~column makes equal sums come out by ascending column; padding (c >= ncand) sorts
+  // last and carries an out-of-range column
+  auto sort_key = [&](int c, uint32_t bits) -> uint64_t {
+    return c < ncand ? (((uint64_t)bits << 32) | (uint32_t)(~(uint32_t)c)) : 0ull;
+  };
   const bool small = np2 <= kSlots * 64;
-  if (small) {
+  if (small) {      // candidates stay in registers; the sort keys are only written if the extraction gives up
 #pragma unroll
     for (int u = 0; u < kSlots; ++u)
       if (u * 64 < np2) {
-        vals[u] = load_one(u * 64 + lane);
+        vals[u] = load_one(u * 64 + lane, true);
         n_others += vals[u] != 0;
       }
   } else {
-    for (int c = lane; c < np2; c += 64) load_one(c);
+    for (int c = lane; c < np2; c += 64) keys[c] = sort_key(c, load_one(c, true));
   }
   for (int c = lane; c < p.nkb; c += 64) flags[c] = 0;
   total = wave_sum(total);
@@ -196,6 +198,10 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
   }
 
   if (!finished) {
+  if (small) {
+    for (int c = lane; c < np2; c += 64) keys[c] = sort_key(c, load_one(c, false));
+    __syncthreads();
+  }
   // ---- bitonic sort, descending
   for (int k = 2; k <= np2; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
