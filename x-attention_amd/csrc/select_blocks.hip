@@ -154,6 +154,9 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
 
   int dropped = 0;
   bool finished = false;
+  // no block sum can exceed a forced key unless the row's total does: otherwise the forced blocks rank first
+  // and a decision does not need the block's own value
+  const bool may_outrank = p.causal && total > key_lo;
   if (small) {
     // ---- extraction: keep pulling out the largest remaining block while the rule says "keep"
 #pragma unroll
@@ -164,6 +167,14 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
         finished = true;
         break;
       }
+      if (!may_outrank) {
+        const double mass = p.causal ? rank_mass(it, n_forced, before, prev_before, prev2_before) : before;
+        if (!(mass < required)) {
+          finished = true;
+          dropped = 1;
+          break;
+        }
+      }
       uint32_t best = 0;
 #pragma unroll
       for (int u = 0; u < kSlots; ++u) best = vals[u] > best ? vals[u] : best;
@@ -173,11 +184,13 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
         best = o > best ? o : best;
       }
       const double best_val = (double)__uint_as_float(best - 1u);
-      const double mass = p.causal ? rank_mass(it, forced_ahead(best_val), before, prev_before, prev2_before) : before;
-      if (!(mass < required)) {
-        finished = true;
-        dropped = 1;
-        break;
+      if (may_outrank) {
+        const double mass = rank_mass(it, forced_ahead(best_val), before, prev_before, prev2_before);
+        if (!(mass < required)) {
+          finished = true;
+          dropped = 1;
+          break;
+        }
       }
       uint32_t col = 0xffffffffu;     // lowest column holding the maximum
 #pragma unroll
@@ -236,10 +249,12 @@ __global__ __launch_bounds__(64) void select_blocks_kernel(SelParams p) {
     const uint32_t col = ~(uint32_t)key;
     if (col < (uint32_t)ncand && (key >> 32) != 0) {
       double mass = before;
-      if (p.causal) {
+      if (may_outrank) {
         const double b1 = rank > 0 ? before - key_value(keys[rank - 1]) : 0.0;
         const double b2 = rank > 1 ? b1 - key_value(keys[rank - 2]) : 0.0;
         mass = rank_mass(rank, forced_ahead(key_value(key)), before, b1, b2);
+      } else if (one_forced) {
+        mass = rank == 0 ? 0.0 : before - key_value(keys[rank - 1]);
       }
       if (mass < required) flags[col] = 1;
       else dropped = 1;
