@@ -205,21 +205,33 @@ __device__ __forceinline__ void mask_tile(f32x16 (&sacc)[4], int kb, int hh, int
     }
 }
 
-// normalises and stores this lane's output row
-__device__ __forceinline__ void store_out(const AttnParams& p, int head, int q_row, int hh, const f32x16 (&oacc)[4], float l_run) {
+// Normalises this wavefront's 32 output rows and stores them through LDS.  Lane (r, hh) holds half of row r in
+// 8-byte pieces; written straight to memory those are 512 sixteen-byte requests per wavefront, and a
+// workgroup's registers and LDS stay allocated until its last store is acknowledged - on lists of a few blocks
+// that wait was a quarter of a workgroup's life.  Staged through the wavefront's own 8 KiB of the K tile
+// (free once the sweep is over), 16 lanes write one 256-byte row: 64 full-line requests.
+__device__ __forceinline__ void store_out(const AttnParams& p, int head, int qb, int wave, int lane, int r, int hh,
+                                          const f32x16 (&oacc)[4], float l_run, char* stage) {
   const float l_tot = half_sum(l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (q_row < p.Lq) {
-    __bf16* dst = p.o + (int64_t)head * p.o_sh + (int64_t)q_row * p.o_sn + hh * 4;
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+  for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack_bf16(oacc[dt][g * 4 + 0] * inv, oacc[dt][g * 4 + 1] * inv);
-        w[1] = pack_bf16(oacc[dt][g * 4 + 2] * inv, oacc[dt][g * 4 + 3] * inv);
-        *reinterpret_cast<u32x2*>(dst + dt * 32 + g * 8) = w;
-      }
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = pack_bf16(oacc[dt][g * 4 + 0] * inv, oacc[dt][g * 4 + 1] * inv);
+      w[1] = pack_bf16(oacc[dt][g * 4 + 2] * inv, oacc[dt][g * 4 + 3] * inv);
+      const int c = dt * 4 + g;                          // 16-byte chunk of the row; XOR-swizzled against bank conflicts
+      *reinterpret_cast<u32x2*>(stage + r * 256 + ((c ^ (r & 15)) << 4) + hh * 8) = w;
+    }
+  // written and read by the same wavefront: the LDS keeps a wavefront's accesses in order, no barrier
+  const int c = lane & 15;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = i * 4 + (lane >> 4);
+    const u32x4 w = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c ^ (row & 15)) << 4));
+    const int q_row = qb * kBlk + wave * 32 + row;
+    if (q_row < p.Lq) *reinterpret_cast<u32x4*>(p.o + (int64_t)head * p.o_sh + (int64_t)q_row * p.o_sn + c * 8) = w;
   }
 }
 
@@ -301,7 +313,8 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     if (kb_next >= 0) copy_tile(vbase, p.v_sn, p.Lk, kb_next, la.voffV, Vs, wave);
     kb = kb_next;
   }
-  store_out(p, head, q_row, hh, oacc, l_run);
+  // the last barrier of the sweep (or the one before it, for an empty list) left both tiles unused
+  store_out(p, head, qb, wave, lane, r, hh, oacc, l_run, Ks + wave * 8192);
 }
 
 }  // namespace xattn
