@@ -63,6 +63,7 @@ def test_attention_entry_points_validate_strides_and_scale_before_launching():
     big = 1 << 23
     assert fwd([ok_strides[0], 128, ok_strides[2], big] + ok_strides[4:]) == -4        # K token stride beyond 2^22
     assert fwd(ok_strides[:5] + [big] + ok_strides[6:]) == -4                          # V token stride
+    assert fwd([ok_strides[0], big] + ok_strides[2:]) == -4                            # Q token stride (a tile like K)
     assert fwd(ok_strides[:3] + [64] + ok_strides[4:]) == -4                           # rows would overlap
     assert fwd(ok_strides, scale=0.0) == -4 and fwd(ok_strides, scale=-1.0) == -4
     assert fwd(ok_strides, scale=float("nan")) == -4

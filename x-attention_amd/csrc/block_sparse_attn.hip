@@ -72,14 +72,6 @@ __device__ __forceinline__ void lane_addressing(const AttnParams& p, int lane, i
     }
 }
 
-// Q^T fragments of one lane's query row (rows past the end repeat the last one; their output is never stored)
-__device__ __forceinline__ void load_q(const __bf16* qbase, int64_t q_sn, int q_row, int Lq, int hh, bf16x8 (&qreg)[8]) {
-  const int row = q_row < Lq ? q_row : Lq - 1;
-  const __bf16* src = qbase + (int64_t)row * q_sn + hh * 8;
-#pragma unroll
-  for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(src + s * 16);
-}
-
 // S^T = K_j Q^T : lane owns query row r, key rows 8g + 4hh + t of each 32-row tile
 __device__ __forceinline__ void qk_tile(const char* Ks, const int (&kaddr)[8], const bf16x8 (&qreg)[8], f32x16 (&sacc)[4]) {
 #pragma unroll
@@ -274,7 +266,6 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   }
 
   bf16x8 qreg[8];   // Q^T fragments stay in registers for the whole sweep
-  load_q(qbase, p.q_sn, q_row, p.Lq, hh, qreg);
   LaneAddr la;
   lane_addressing(p, lane, wave, la);
 
@@ -287,10 +278,22 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   float l_run = 0.f;         // this lane's share of the running row sum
 
   int kb = 0;
-  if (n_blocks > 0) {
-    kb = kHasList ? clamp_block(list[0], p.nkb) : 0;
-    copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
-    copy_tile(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
+  {
+    // The q-block is a tile like any other: copied row-wise (full lines) into the V tile, where each wavefront's
+    // eighth-of-a-tile copies are its own 32 query rows, and read back as fragments before V_0 is requested.
+    int voffQ[8];
+    tile_offsets(p.q_sn, lane, wave, voffQ);
+    copy_tile(qbase, p.q_sn, p.Lq, qb, voffQ, Vs, wave);
+    if (n_blocks > 0) {
+      kb = kHasList ? clamp_block(list[0], p.nkb) : 0;
+      copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
+    }
+    wait_vm0();
+#pragma unroll
+    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(Vs + wave * 8192 + la.kaddr[s]);
+    __builtin_amdgcn_s_waitcnt(0xC07F);      // the fragments are in registers before V_0 may overwrite them
+    asm volatile("" ::: "memory");
+    if (n_blocks > 0) copy_tile(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
   }
   wait_vm0();
   __syncthreads();                         // K_0 (and V_0) landed and visible
@@ -341,7 +344,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   for (int64_t s : strides)
     if (s % 8) return XATTN_ERR_ALIGN;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return XATTN_ERR_ALIGN;
-  if (!tile_stride_ok(k_stride_n) || !tile_stride_ok(v_stride_n) || q_stride_n < kHeadDim || o_stride_n < kHeadDim)
+  if (!tile_stride_ok(k_stride_n) || !tile_stride_ok(v_stride_n) || !tile_stride_ok(q_stride_n) || o_stride_n < kHeadDim)
     return XATTN_ERR_SHAPE;
   if (!scale_ok(softmax_scale)) return XATTN_ERR_SHAPE;
 
