@@ -20,7 +20,12 @@
 // issued one k-step ahead of the MFMAs that consume them.  The copy of the next
 // K tile overlaps softmax and P.V, the copy of the next V tile overlaps Q.K^T.
 // Two workgroups fit per CU (64 KiB LDS each) so one's softmax overlaps the
-// other's MFMA.
+// other's MFMA.  The query block enters and the output block leaves through
+// the same LDS tiles as full 256-byte rows (the q-block is copied like a K
+// tile before V_0 is requested; the output is staged in the K tile after the
+// sweep): row-per-lane accesses to global memory would be hundreds of partial
+// line requests per wavefront, and a workgroup keeps its registers and LDS
+// until the last of its stores is acknowledged.
 #include "attn_tiles.h"
 #include "xattn_hip.h"
 
