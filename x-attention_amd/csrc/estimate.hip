@@ -14,7 +14,9 @@
 //    keys, exponentiates against that local maximum and adds up groups of
 //    block_size/S keys.  It writes, per (query row, 128-key tile), the local
 //    maximum and sum, and per (query row, key block) the partial sum - 1/S of
-//    the score matrix, in fp32 - never the scores themselves.
+//    the score matrix, in fp32 - never the scores themselves.  One workgroup
+//    per CU works through its share of the tiles with the copy pipeline
+//    running on across tile boundaries.
 //  kernel 2 (estimate_normalize_kernel): per query row, combines the tile
 //    maxima/sums into the row's softmax statistics, rescales the partial sums
 //    and adds the block_size/S rows of each query block.
