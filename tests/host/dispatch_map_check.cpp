@@ -1,7 +1,6 @@
-// Host-only check of the attention kernels' workgroup -> (head, q-block) maps
-// (one unit per workgroup for the block-mass profiler, a pair of units for the
-// attention kernel): over a launch of grid_for() / pair_grid() ids every
-// (head, q-block) of the range must be produced exactly once and nothing else.  Prints one line per case; exit
+// Host-only check of the attention kernels' workgroup -> (head, q-block) map:
+// over a launch of grid_for() ids every (head, q-block) of the range must be
+// produced exactly once and nothing else.  Prints one line per case; exit
 // status 0 when all hold.  No GPU call is made.
 #include <cstdio>
 #include <vector>
@@ -51,47 +50,6 @@ int main() {
     std::printf("H=%d Hkv=%d q-blocks [%d,%d): grid %ld missing %ld twice %ld stray %ld mixed-units %ld\n", H, Hkv, b, e,
                 grid, missing, twice, stray, mixed);
     bad += (missing || twice || stray || mixed) ? 1 : 0;
-
-    // The pair map of the attention kernel: every (head, q-block) in exactly one pair, both units of a
-    // pair on one KV head, and the 32 ids that reach an XCD one after the other on one KV head.
-    const long pgrid = (long)xattn::pair_grid(H, Hkv, e - b);
-    const long n_units = (long)(H / Hkv) * (e - b);
-    std::vector<int> pseen((size_t)H * (e - b), 0);
-    long pstray = 0, pmixed = 0;
-    for (long id = 0; id < pgrid; ++id) {
-      int kvh = -1;
-      int64_t u0 = -1;
-      if (!xattn::map_pair((int)id, H, Hkv, e - b, &kvh, &u0)) continue;
-      for (int g = 0; g < 2; ++g) {
-        if (u0 + g >= n_units) continue;
-        int head = -1, qb = -1;
-        xattn::pair_unit(u0 + g, kvh, H, Hkv, e, &head, &qb);
-        if (head < 0 || head >= H || qb < b || qb >= e || head / (H / Hkv) != kvh) {
-          ++pstray;
-          continue;
-        }
-        ++pseen[(size_t)head * (e - b) + (qb - b)];
-      }
-    }
-    for (long u = 0; u * 256 < pgrid; ++u)
-      for (int x = 0; x < 8; ++x) {
-        int kv = -1;
-        for (int w = 0; w < 32; ++w) {
-          int kvh;
-          int64_t u0;
-          if (!xattn::map_pair((int)(u * 256 + w * 8 + x), H, Hkv, e - b, &kvh, &u0)) continue;
-          if (kv >= 0 && kvh != kv) ++pmixed;
-          kv = kvh;
-        }
-      }
-    long pmissing = 0, ptwice = 0;
-    for (int v : pseen) {
-      pmissing += v == 0;
-      ptwice += v > 1;
-    }
-    std::printf("  pairs: grid %ld pair-missing %ld pair-twice %ld pair-stray %ld pair-mixed %ld\n", pgrid, pmissing, ptwice,
-                pstray, pmixed);
-    bad += (pmissing || ptwice || pstray || pmixed) ? 1 : 0;
   }
   return bad ? 1 : 0;
 }

@@ -25,4 +25,3 @@ def test_every_head_and_q_block_is_dispatched_exactly_once(tmp_path):
     print(run.stdout)
     assert run.returncode == 0, run.stdout
     assert run.stdout.count("missing 0 twice 0 stray 0 mixed-units 0") >= 16
-    assert run.stdout.count("pair-missing 0 pair-twice 0 pair-stray 0 pair-mixed 0") >= 16

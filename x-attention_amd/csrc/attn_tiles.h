@@ -33,62 +33,32 @@ __device__ __forceinline__ void copy_tile(const __bf16* base, int64_t sn, int le
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(tile + (wave * 8 + i) * 1024), 16, voff[i], 0, 0, 0);
 }
 
-// The same copy with the per-lane offsets held in four registers: instruction i moves rows
-// 4*(8*wave + i) + lane/16, whose swizzle term depends on i % 4 only (swz(row) = ((lane/16) << 2) | (i % 4)),
-// so voff[i % 4] holds rows 32*wave + lane/16 with that term and the remaining i * 4 rows go into the
-// instruction's scalar offset (row4 = bytes of four token rows).
-//
-// Issued from one assembly block, M0 (the LDS destination) included: the compiler makes every LDS read that
-// follows a buffer load into LDS it knows of wait for that load (the two might alias), which would expose the
-// whole copy latency at the next fragment read.  Loads issued this way are not counted by the compiler, so
-// the caller waits for them itself (wait_vm0) before the barrier that publishes the tile; loads return in
+// The same copy issued from one assembly block, M0 (the LDS destination) included.  The compiler makes the
+// transposing LDS reads wait for every buffer load into LDS it knows of (the two might alias), which exposes
+// the whole copy latency at the next fragment read; loads issued this way are not counted by the compiler, so
+// the caller waits for them itself (wait_vm0) before the barrier that publishes the tile.  Loads return in
 // order, so the compiler's own vmcnt waits for its own loads stay sufficient.
-__device__ __forceinline__ void copy_tile4(const __bf16* base, int64_t sn, int len, int kb, const int (&voff)[4],
-                                           int row4, char* tile, int wave) {
+__device__ __forceinline__ void copy_tile_async(const __bf16* base, int64_t sn, int len, int kb, const int (&voff)[8],
+                                                char* tile, int wave) {
   const int rows_left = len - kb * kBlk;
   const int rows = rows_left < kBlk ? rows_left : kBlk;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)(base + (int64_t)kb * kBlk * sn), 0, (int)((int64_t)rows * sn * 2), 0x00020000);
-  const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr_t)(tile + wave * 8 * 1024);
+  const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(tile + wave * 8 * 1024));
   asm volatile(
-      "s_mov_b32 m0, %[dst]\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v0], %[rs], 0 offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v1], %[rs], %[s1] offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v2], %[rs], %[s2] offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v3], %[rs], %[s3] offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v0], %[rs], %[s4] offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v1], %[rs], %[s5] offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v2], %[rs], %[s6] offen lds\n\t"
-      "s_add_u32 m0, m0, 0x400\n\t"
-      "s_nop 0\n\t"
-      "buffer_load_dwordx4 %[v3], %[rs], %[s7] offen lds"
+      "s_mov_b32 m0, %[dst]\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v0], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v1], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v2], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v3], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v4], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v5], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v6], %[rs], 0 offen lds\n\ts_add_u32 m0, m0, 0x400\n\ts_nop 0\n\t"
+      "buffer_load_dwordx4 %[v7], %[rs], 0 offen lds"
       :
       : [dst] "s"(dst), [rs] "s"(rsrc), [v0] "v"(voff[0]), [v1] "v"(voff[1]), [v2] "v"(voff[2]), [v3] "v"(voff[3]),
-        [s1] "s"(row4), [s2] "s"(2 * row4), [s3] "s"(3 * row4), [s4] "s"(4 * row4), [s5] "s"(5 * row4),
-        [s6] "s"(6 * row4), [s7] "s"(7 * row4)
+        [v4] "v"(voff[4]), [v5] "v"(voff[5]), [v6] "v"(voff[6]), [v7] "v"(voff[7])
       : "memory", "m0", "scc");
-}
-
-__device__ __forceinline__ void tile_offsets4(int64_t sn, int lane, int wave, int (&voff)[4]) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = 4 * (wave * 8) + (lane >> 4);
-    const int c = (lane & 15) ^ swz(4 * i + (lane >> 4));
-    voff[i] = (int)(row * sn * 2) + (c << 4);
-  }
 }
 
 __device__ __forceinline__ void tile_offsets(int64_t sn, int lane, int wave, int (&voff)[8]) {
@@ -149,48 +119,6 @@ inline int64_t grid_for(int H, int Hkv, int n_qblocks) {
   const DispatchShape d = dispatch_shape(H, Hkv);
   const int64_t runs = (n_qblocks + d.unit_rows - 1) / d.unit_rows;
   return ((runs * d.n_groups + 7) / 8 * 8) * kUnit;
-}
-
-// Dispatch of the attention kernel proper, whose workgroups (eight wavefronts,
-// one per CU) each take TWO (head, q-block) units that read the same KV head.
-// The units of a KV head are numbered u = from_end * G + g (G query heads per
-// KV head, g the head inside its group, from_end counted from the last q-block
-// of the launch: longest rows first when causal); workgroup m of that KV head
-// takes units 2m and 2m + 1 - two heads of the group on one q-block when G is
-// even, else whatever neighbours the numbering gives (for G = 1 two adjacent
-// q-blocks of one head).  The 32 ids that land on one XCD one after the other
-// are 32 consecutive pairs of one KV head; such windows go to the XCDs in turn
-// and the KV head rotates from one run of windows to the next.
-constexpr int kPairWindow = 32;          // workgroups resident on one XCD (32 CUs x 1)
-
-// Returns false for ids that carry no work; *first_unit is even, and unit
-// *first_unit + 1 exists only when it is below G * n_qblocks.
-__host__ __device__ inline bool map_pair(int id, int H, int Hkv, int n_qblocks, int* kvh, int64_t* first_unit) {
-  if (id < 0) return false;
-  const int64_t units = (int64_t)(H / Hkv) * n_qblocks;
-  const int64_t pairs = (units + 1) / 2;
-  const int x = id & 7, s = id >> 3;
-  const int window = (s / kPairWindow) * 8 + x, w = s % kPairWindow;
-  const int run = window / Hkv;
-  const int64_t m = (int64_t)run * kPairWindow + w;
-  if (m >= pairs) return false;
-  *kvh = (window % Hkv + run) % Hkv;
-  *first_unit = 2 * m;
-  return true;
-}
-
-// (head, q-block) of unit u of KV head kvh in a launch over q-blocks [qb_begin, qb_end)
-__host__ __device__ inline void pair_unit(int64_t u, int kvh, int H, int Hkv, int qb_end, int* head, int* qb) {
-  const int G = H / Hkv;
-  *head = kvh * G + (int)(u % G);
-  *qb = qb_end - 1 - (int)(u / G);
-}
-
-// grid size of a launch over n_qblocks q-blocks
-inline int64_t pair_grid(int H, int Hkv, int n_qblocks) {
-  const int64_t pairs = ((int64_t)(H / Hkv) * n_qblocks + 1) / 2;
-  const int64_t runs = (pairs + kPairWindow - 1) / kPairWindow;
-  return ((runs * Hkv + 7) / 8 * 8) * kPairWindow;
 }
 
 // Token strides of K and V the tile copies can address (byte offsets inside a

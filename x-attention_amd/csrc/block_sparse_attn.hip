@@ -18,7 +18,9 @@
 // the buffer resource and arrive as zeros.  K fragments are read with
 // ds_read_b128, V^T fragments with the transposing ds_read_b64_tr_b16, both
 // issued one k-step ahead of the MFMAs that consume them.  The copy of the next
-// K tile overlaps softmax and P.V, the copy of the next V tile overlaps Q.K^T.
+// K tile overlaps softmax and P.V, the copy of the next V tile overlaps Q.K^T
+// (both issued from assembly, see copy_tile_async: the compiler would make the
+// transposing reads wait for every copy it knows of).
 // Two workgroups fit per CU (64 KiB LDS each) so one's softmax overlaps the
 // other's MFMA.  The query block enters and the output block leaves through
 // the same LDS tiles as full 256-byte rows (the q-block is copied like a K
@@ -50,50 +52,49 @@ struct AttnParams {
 
 __device__ __forceinline__ int clamp_block(int kb, int nkb) { return kb < 0 ? 0 : (kb < nkb ? kb : nkb - 1); }
 
-// Per-lane addressing that does not depend on the (head, q-block) being worked on.  Kept to a few
-// registers; the remaining terms are constants folded into the instructions' offsets or XORed in on use
-// (every tile starts at a multiple of 32 KiB, so XORs below bit 12 never carry).
+// Per-lane addressing that does not depend on the (head, q-block) being worked on.
 struct LaneAddr {
-  int voff[4];              // tile copy (V tiles for group 0, K tiles for group 1): byte offset of the lane's row in
-                            // copy instruction i is voff[i % 4] + i * 4 rows
-  int row4;                 // bytes of four token rows of that tensor (the scalar part of a copy's offset)
-  int kaddr;                // K fragment of k-step s, key tile nt: kaddr ^ (s << 5), + nt * 8192
-  int vaddr;                // V^T fragment of k-step ks, half a, feature tile dt: vaddr ^ (dt << 6) ^ (a * 0x820), + ks * 4096
+  int voffK[8], voffV[8];   // tile copy: byte offsets of the lane's rows
+  int kaddr[8];             // K fragment (k-step s, key tile nt): row nt*32 + r, logical chunk 2s + hh
+  int vaddr[4][2];          // V^T fragment (k-step ks, half a, feature tile dt)
 };
 
-// LDS address of a K fragment: row nt*32 + r, logical chunk 2s + hh of the swizzled layout
-//   r*256 + (((2s + hh) ^ swz(r)) << 4) = (r*256 + ((hh ^ swz(r)) << 4)) ^ (s << 5)
-// and of a transposed V fragment: the transposing read hands lane l the feature dt*32 + (l % 32) of keys
-// 16ks + 8a + 4hh + {0..3}; as a source lane it points at key e = (l%16)/4 of that quad, features
-// dt*32 + 16*((l/16)%2) + 4*(l%4) .. +3, i.e. row = 8a + 4hh + e, chunk c = 4dt + 2g2 + (j >> 1), where
-// swz(row) = (e << 2) | (2a + hh), so that
-//   row*256 + ((c ^ swz(row)) << 4) + (j & 1)*8 = base ^ (dt << 6) ^ (a << 5) ^ (a << 11)
-__device__ __forceinline__ void lane_addressing(int64_t sn, int lane, int wq, LaneAddr& a) {
+__device__ __forceinline__ void lane_addressing(const AttnParams& p, int lane, int wave, LaneAddr& a) {
   const int r = lane & 31, hh = lane >> 5;
-  tile_offsets4(sn, lane, wq, a.voff);
-  a.row4 = (int)(4 * sn * 2);
-  a.kaddr = r * 256 + ((hh ^ swz(r)) << 4);
+  tile_offsets(p.k_sn, lane, wave, a.voffK);
+  tile_offsets(p.v_sn, lane, wave, a.voffV);
+#pragma unroll
+  for (int s = 0; s < 8; ++s) a.kaddr[s] = r * 256 + (((2 * s + hh) ^ swz(r)) << 4);
+  // the transposing read hands lane l the feature dt*32 + (l % 32) of keys
+  // 16ks + 8a + 4hh + {0..3}; as a source lane it points at key e = (l%16)/4 of
+  // that quad, features dt*32 + 16*((l/16)%2) + 4*(l%4) .. +3.
   const int e = (lane & 15) >> 2, j = lane & 3, g2 = (lane >> 4) & 1;
-  const int row = 4 * hh + e;
-  a.vaddr = row * 256 + (((2 * g2 + (j >> 1)) ^ swz(row)) << 4) + (j & 1) * 8;
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int row = 8 * h2 + 4 * hh + e;                       // + 16*ks
+      const int c = dt * 4 + 2 * g2 + (j >> 1);
+      a.vaddr[dt][h2] = row * 256 + ((c ^ swz(row)) << 4) + (j & 1) * 8;
+    }
 }
 
 // S^T = K_j Q^T : lane owns query row r, key rows 8g + 4hh + t of each 32-row tile
-__device__ __forceinline__ void qk_tile(const char* Ks, int kaddr, const bf16x8 (&qreg)[8], f32x16 (&sacc)[4]) {
+__device__ __forceinline__ void qk_tile(const char* Ks, const int (&kaddr)[8], const bf16x8 (&qreg)[8], f32x16 (&sacc)[4]) {
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) sacc[i][v] = 0.f;
   bf16x8 kf[2][4];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) kf[0][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr + nt * 8192);
+  for (int nt = 0; nt < 4; ++nt) kf[0][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[0] + nt * 8192);
   __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
     if (s < 7) {
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
-        kf[(s + 1) & 1][nt] = *reinterpret_cast<const bf16x8*>(Ks + (kaddr ^ ((s + 1) << 5)) + nt * 8192);
+        kf[(s + 1) & 1][nt] = *reinterpret_cast<const bf16x8*>(Ks + kaddr[s + 1] + nt * 8192);
     }
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) sacc[nt] = mfma32(kf[s & 1][nt], qreg[s], sacc[nt]);
@@ -149,14 +150,14 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[4], f32x16 (&oacc)[4
 }
 
 // O^T += V_j^T P^T
-__device__ __forceinline__ void pv_tile(const char* Vs, int vaddr, const bf16x8 (&pfrag)[8], f32x16 (&oacc)[4]) {
+__device__ __forceinline__ void pv_tile(const char* Vs, const int (&vaddr)[4][2], const bf16x8 (&pfrag)[8], f32x16 (&oacc)[4]) {
   i16x4 vf[2][4][2];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
     for (int a = 0; a < 2; ++a)
       vf[0][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (__attribute__((address_space(3))) i16x4*)(Vs + (vaddr ^ (dt << 6) ^ (a * 0x820))));
+          (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a]));
   __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
@@ -166,7 +167,7 @@ __device__ __forceinline__ void pv_tile(const char* Vs, int vaddr, const bf16x8 
 #pragma unroll
         for (int a = 0; a < 2; ++a)
           vf[(ks + 1) & 1][dt][a] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) i16x4*)(Vs + (vaddr ^ (dt << 6) ^ (a * 0x820)) + (ks + 1) * 4096));
+              (__attribute__((address_space(3))) i16x4*)(Vs + vaddr[dt][a] + (ks + 1) * 4096));
     }
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
@@ -235,213 +236,95 @@ __device__ __forceinline__ void store_out(const AttnParams& p, int head, int qb,
 
 typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
-constexpr int kNoTile = 0x7fffffff;
-
-// One (head, q-block) of the pair a workgroup works on (all scalar).
-struct Unit {
-  int head, qb;
-  int n;                 // entries of its column list / visible blocks; 0 for the missing partner of an odd last unit
-  const_i32_ptr list;    // ascending k-block ids (kHasList only)
-};
-
-// A step of the merged walk over the two units' ascending lists: key block t (kNoTile past the end), whether
-// the wavefront's own unit visits it, and whether anybody does.
-struct Step {
-  int t;
-  bool mine;
-};
-
-// Workgroup-level barrier that leaves the tile copies in flight alone (only LDS traffic is drained).
-__device__ __forceinline__ void phase_barrier() {
-  __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
-
 // kHasList = false is the dense baseline (its own symbol, so profiles tell the two apart)
-//
-// Eight wavefronts: group 0 (wavefronts 0-3) works on the first unit of the pair, group 1 (4-7) on the second;
-// wavefront wq of either group owns query rows 32 wq .. +31 of its unit's q-block and sits on SIMD wq, so each
-// SIMD holds one wavefront of each group.  Both groups run the same loop over the merged block walk -
-//     matrix phase:  O^T += V_{j-1}^T P^T,  S^T = K_j Q^T      (64 MFMAs)
-//     vector phase:  mask, online softmax, bf16 packing of tile j
-// - separated by workgroup barriers, with group 1 started one phase late: whenever one wavefront of a SIMD
-// issues MFMAs the other does the exponentials, instead of two workgroups drifting against each other.
-// K and V tiles are shared by the groups, double-buffered (4 x 32 KiB): tile j is read by group 0 in phase
-// 2j (K) / 2j+2 (V) and by group 1 one phase later.  Copies are issued at the start of even phases (V_j by
-// group 0, K_{j+2} by group 1, each wavefront a quarter of the tile) and awaited at the end of the next odd
-// phase, two phases later.  A unit that does not visit a block of the walk idles through its two phases.
 template <bool kHasList>
-__global__ __launch_bounds__(512) void block_sparse_fwd_kernel(AttnParams p) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
-  char* const Kb = lds;                       // K tiles: [2][kTileBytes]
-  char* const Vb = lds + 2 * kTileBytes;      // V tiles: [2][kTileBytes]
+__global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(1024))) char Ks[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) char Vs[kTileBytes];
 
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int grp = wave >> 2, wq = wave & 3;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
 
-  int kvh;
-  int64_t u0;
-  if (!map_pair(blockIdx.x, p.H, p.Hkv, p.qb_end - p.qb_begin, &kvh, &u0)) return;
-  const int64_t n_units = (int64_t)(p.H / p.Hkv) * (p.qb_end - p.qb_begin);
-
-  const bool mine_exists = u0 + grp < n_units;
-  auto make_unit = [&](int g) -> Unit {
-    Unit u;
-    const bool exists = u0 + g < n_units;
-    pair_unit(exists ? u0 + g : u0, kvh, p.H, p.Hkv, p.qb_end, &u.head, &u.qb);
-    const int q_last = (u.qb * kBlk + kBlk - 1 < p.Lq ? u.qb * kBlk + kBlk - 1 : p.Lq - 1) + p.kv_off;
-    int visible = p.causal ? (q_last < 0 ? 0 : q_last / kBlk + 1) : p.nkb;
-    visible = visible < p.nkb ? visible : p.nkb;
-    u.list = nullptr;
-    if (kHasList) {
-      // the column lists are read through the scalar cache (uniform, read-only), so that fetching the next
-      // block ids never waits on the tile copies in flight
-      const int64_t slot = (int64_t)u.head * p.idx_rows + (u.qb - p.idx_row0);
-      u.list = (const_i32_ptr)(uintptr_t)(p.col_idx + slot * p.idx_pitch);
-      int n = ((const_i32_ptr)(uintptr_t)p.col_cnt)[slot];
-      u.n = n < 0 ? 0 : (n > p.idx_pitch ? (int)p.idx_pitch : n);
-    } else {
-      u.n = visible;
-    }
-    if (!exists) u.n = 0;
-    return u;
-  };
-  const Unit un0 = make_unit(0), un1 = make_unit(1);
-  const int head = grp ? un1.head : un0.head, qb = grp ? un1.qb : un0.qb;
+  int head, qb;
+  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, p.qb_begin, p.qb_end, &head, &qb)) return;
+  const int kvh = head / (p.H / p.Hkv);
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
   const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
-  const int q_row = qb * kBlk + wq * 32 + r;            // this lane's query token
+
+  const int q_row = qb * kBlk + wave * 32 + r;          // this lane's query token
   const int q_pos = q_row + p.kv_off;                   // its position on the key axis
-
-  LaneAddr la;
-  lane_addressing(grp ? p.k_sn : p.v_sn, lane, wq, la);
-
-  // the q-block is a tile like any other: copied row-wise (full lines) into a V tile - group g's into V
-  // tile g, each wavefront its own 32 query rows - and read back as fragments before that tile's first V
-  // copy is issued (V_0 by group 0's wavefronts, row for row over their own query rows; V_1 after the
-  // barrier that follows group 1's fragment reads)
+  int n_blocks;
+  // the column list is read through the scalar cache (uniform, read-only), so that
+  // fetching the next block id never waits on the tile copies in flight
+  const_i32_ptr list = nullptr;
   {
-    int voffQ[8];
-    tile_offsets(p.q_sn, lane, wq, voffQ);
-    if (mine_exists) copy_tile(qbase, p.q_sn, p.Lq, qb, voffQ, Vb + grp * kTileBytes, wq);
+    const int q_last = (qb * kBlk + kBlk - 1 < p.Lq ? qb * kBlk + kBlk - 1 : p.Lq - 1) + p.kv_off;
+    int visible = p.causal ? (q_last < 0 ? 0 : q_last / kBlk + 1) : p.nkb;
+    visible = visible < p.nkb ? visible : p.nkb;
+    if (kHasList) {
+      const int64_t slot = (int64_t)head * p.idx_rows + (qb - p.idx_row0);
+      list = (const_i32_ptr)(uintptr_t)(p.col_idx + slot * p.idx_pitch);
+      n_blocks = ((const_i32_ptr)(uintptr_t)p.col_cnt)[slot];
+      n_blocks = n_blocks < 0 ? 0 : (n_blocks > p.idx_pitch ? (int)p.idx_pitch : n_blocks);
+    } else {
+      n_blocks = visible;
+    }
   }
 
-  // merged walk: e0 / e1 are the head entries of the two lists, f0 / f1 the entries after them (loaded a
-  // step before they are needed)
-  int i0 = 0, i1 = 0;
-  auto entry = [&](const Unit& u, int i) -> int {
-    if (i >= u.n) return kNoTile;
-    return kHasList ? clamp_block(u.list[i], p.nkb) : i;
-  };
-  int e0 = entry(un0, 0), f0 = entry(un0, 1), e1 = entry(un1, 0), f1 = entry(un1, 1);
-  auto advance = [&]() -> Step {
-    Step s;
-    s.t = e0 < e1 ? e0 : e1;
-    const bool in0 = s.t != kNoTile && e0 == s.t, in1 = s.t != kNoTile && e1 == s.t;
-    if (in0) {
-      e0 = f0;
-      ++i0;
-      f0 = entry(un0, i0 + 1);
-    }
-    if (in1) {
-      e1 = f1;
-      ++i1;
-      f1 = entry(un1, i1 + 1);
-    }
-    s.mine = grp ? in1 : in0;
-    return s;
-  };
-  Step prev, cur, nxt, nxt2;
-  prev.t = kNoTile;
-  prev.mine = false;
-  cur = advance();
-  nxt = advance();
-  nxt2 = advance();
-
-  // K_0 by group 0, K_1 by group 1 (from then on group 1 copies K_{j+2} in its vector phase of tile j)
-  {
-    int voffK0[8];
-    tile_offsets(p.k_sn, lane, wq, voffK0);
-    const int first = grp ? nxt.t : cur.t;
-    if (first != kNoTile) copy_tile(kbase, p.k_sn, p.Lk, first, voffK0, Kb + grp * kTileBytes, wq);
-  }
-  wait_vm0();
   bf16x8 qreg[8];   // Q^T fragments stay in registers for the whole sweep
-#pragma unroll
-  for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(Vb + grp * kTileBytes + wq * 8192 + (la.kaddr ^ (s << 5)));
-  phase_barrier();  // K_0, K_1 visible; every wavefront holds its Q fragments
+  LaneAddr la;
+  lane_addressing(p, lane, wave, la);
 
-  f32x16 oacc[4], sacc[4];
+  f32x16 oacc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      oacc[i][v] = 0.f;
-      sacc[i][v] = 0.f;
-    }
-  bf16x8 pfrag[8];
-#pragma unroll
-  for (int s = 0; s < 8; ++s)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) pfrag[s][e] = (__bf16)0.f;
+    for (int v = 0; v < 16; ++v) oacc[i][v] = 0.f;
   float m_run = -INFINITY;   // running row maximum, already multiplied by scale_log2
   float l_run = 0.f;         // this lane's share of the running row sum
 
-  if (grp) phase_barrier();  // group 1 runs one phase behind group 0
-
-  for (int j = 0;; ++j) {
-    const bool last = cur.t == kNoTile;      // iteration n: only the P.V of tile n-1 is left
-    char* const Kt = Kb + (j & 1) * kTileBytes;
-    char* const Vt = Vb + (j & 1) * kTileBytes;
-    char* const Vp = Vb + ((j + 1) & 1) * kTileBytes;   // V_{j-1}
-
-    // ---- matrix phase (group 0: phase 2j, group 1: phase 2j+1)
-    if (!grp && !last) copy_tile4(vbase, p.v_sn, p.Lk, cur.t, la.voff, la.row4, Vt, wq);
-    __builtin_amdgcn_s_setprio(2);
-    if (prev.mine) pv_tile(Vp, la.vaddr, pfrag, oacc);
-    if (cur.mine) {
-      qk_tile(Kt, la.kaddr, qreg, sacc);
-    } else {
-      // (defining the scores on this path too tells the register allocator that nothing of the last tile's
-      // scores is alive here: they and the packed probabilities then share registers)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) sacc[i][v] = 0.f;
+  int kb = 0;
+  {
+    // The q-block is a tile like any other: copied row-wise (full lines) into the V tile, where each wavefront's
+    // eighth-of-a-tile copies are its own 32 query rows, and read back as fragments before V_0 is requested.
+    int voffQ[8];
+    tile_offsets(p.q_sn, lane, wave, voffQ);
+    copy_tile(qbase, p.q_sn, p.Lq, qb, voffQ, Vs, wave);
+    if (n_blocks > 0) {
+      kb = kHasList ? clamp_block(list[0], p.nkb) : 0;
+      copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
     }
-    __builtin_amdgcn_s_setprio(0);
-    if (grp) wait_vm0();                     // end of an odd phase: the copies of the last even phase landed
-    phase_barrier();
-
-    // ---- vector phase (group 0: phase 2j+1, group 1: phase 2j+2); nothing but the barrier in the last iteration
-    if (grp && nxt2.t != kNoTile) copy_tile4(kbase, p.k_sn, p.Lk, nxt2.t, la.voff, la.row4, Kt, wq);
-    if (cur.mine) {
-      const int kb = cur.t;
-      const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
-      if (need_mask) mask_tile(sacc, kb, hh, q_pos, p.Lk, p.causal);
-      softmax_tile(sacc, oacc, m_run, l_run, p.scale_log2, pfrag);
-    } else {
+    wait_vm0();
 #pragma unroll
-      for (int s = 0; s < 8; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pfrag[s][e] = (__bf16)0.f;
-    }
-    if (!grp) wait_vm0();
-    phase_barrier();
-    if (last) break;       // (the loop leaves at its end: an exit in the middle made the compiler keep two copies of the accumulators)
-    prev = cur;
-    cur = nxt;
-    nxt = nxt2;
-    nxt2 = advance();
+    for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const bf16x8*>(Vs + wave * 8192 + la.kaddr[s]);
+    __builtin_amdgcn_s_waitcnt(0xC07F);      // the fragments are in registers before V_0 may overwrite them
+    asm volatile("" ::: "memory");
+    if (n_blocks > 0) copy_tile_async(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
   }
-  // Group 0 is done one phase before group 1.  Every K tile has been read (the last in phase 2n-1) and no
-  // copy is in flight, so each wavefront stages its rows in its own 8 KiB of the K tiles.
-  if (mine_exists) store_out(p, head, qb, wq, lane, r, hh, oacc, l_run, Kb + wave * 8192);
-  if (!grp) phase_barrier();   // pairs with group 1's last barrier: both groups pass the same number
+  wait_vm0();
+  __syncthreads();                         // K_0 (and V_0) landed and visible
+
+  for (int j = 0; j < n_blocks; ++j) {
+    const int kb_next = (j + 1 < n_blocks) ? (kHasList ? clamp_block(list[j + 1], p.nkb) : j + 1) : -1;
+    f32x16 sacc[4];
+    qk_tile(Ks, la.kaddr, qreg, sacc);
+    wait_vm0();
+    __syncthreads();                       // everyone is done with K_j; V_j landed and visible
+    if (kb_next >= 0) copy_tile_async(kbase, p.k_sn, p.Lk, kb_next, la.voffK, Ks, wave);
+
+    const bool need_mask = (kb * kBlk + kBlk > p.Lk) || (p.causal && kb * kBlk + kBlk - 1 > qb * kBlk + p.kv_off);
+    if (need_mask) mask_tile(sacc, kb, hh, q_pos, p.Lk, p.causal);
+    bf16x8 pfrag[8];
+    softmax_tile(sacc, oacc, m_run, l_run, p.scale_log2, pfrag);
+    pv_tile(Vs, la.vaddr, pfrag, oacc);
+    wait_vm0();
+    __syncthreads();                       // everyone is done with V_j; K_{j+1} landed and visible
+    if (kb_next >= 0) copy_tile_async(vbase, p.v_sn, p.Lk, kb_next, la.voffV, Vs, wave);
+    kb = kb_next;
+  }
+  // the last barrier of the sweep (or the one before it, for an empty list) left both tiles unused
+  store_out(p, head, qb, wave, lane, r, hh, oacc, l_run, Ks + wave * 8192);
 }
 
 }  // namespace xattn
@@ -495,18 +378,13 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   p.idx_row0 = idx_row0;
   p.qb_begin = q_block_begin;
   p.qb_end = q_block_end;
-  const int64_t grid = pair_grid(p.H, p.Hkv, q_block_end - q_block_begin);
+  const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
-  const void* kernel = col_idx ? reinterpret_cast<const void*>(&block_sparse_fwd_kernel<true>)
-                               : reinterpret_cast<const void*>(&block_sparse_fwd_kernel<false>);
-  constexpr int kLds = 4 * kTileBytes;   // two K and two V tiles: one workgroup per CU
-  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds) != hipSuccess)
-    return XATTN_ERR_LAUNCH;
   if (col_idx)
-    hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(512), kLds,
+    hipLaunchKernelGGL(block_sparse_fwd_kernel<true>, dim3((unsigned)grid), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
   else
-    hipLaunchKernelGGL(block_sparse_fwd_kernel<false>, dim3((unsigned)grid), dim3(512), kLds,
+    hipLaunchKernelGGL(block_sparse_fwd_kernel<false>, dim3((unsigned)grid), dim3(256), 0,
                        static_cast<hipStream_t>(stream), p);
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
 }
