@@ -160,6 +160,36 @@ int xattn_select_blocks(const float* block_sums, const double* tau_per_head, uin
                         void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Estimate and selection in one call, for callers that want the column lists
+ * (or the mask) and not the block sums - what the operator does at
+ * xattn/src/Xattention.py:358-385, which never looks at attn_sums.  Same
+ * arithmetic and results as xattn_estimate_block_sums followed by
+ * xattn_select_blocks over the q-block rows of chunks [chunk_begin, chunk_end)
+ * (replaces xattn/src/kernels.py:68-90 + xattn/src/utils.py:87-146 for that
+ * use): the normalisation pass leaves each q-block row's block sums in LDS and
+ * one wavefront selects from them there, so the sums make no round trip through
+ * memory.  Arguments are those of the two entry points (the selection's geometry
+ * - diagonal offset, list_cols, kv_off_tokens, blocks_per_chunk - follows from
+ * the lengths); `block_sums` may be null, or receive the sums as well.  The
+ * default reshape's row subsampling (kdb) is not available here, and padded key
+ * lengths beyond 8192 blocks are refused with XATTN_ERR_SHAPE (use the two
+ * entry points).  mask, col_idx/col_cnt, window_row0/window_rows as for
+ * xattn_select_blocks.  `stages`: 3 runs both passes; 1 only the MFMA pass
+ * (partial sums into the workspace), 2 only the normalise-and-select pass over a
+ * workspace a stages = 1 call with the same arguments filled - for callers that
+ * want an event or another stream between the two.
+ */
+int xattn_estimate_select(const void* q, const void* k, float* block_sums, void* workspace,
+                          size_t workspace_bytes, int num_heads, int num_kv_heads, int q_len, int k_len,
+                          int head_dim, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
+                          int64_t k_stride_n, int stride, int block_size, int chunk_size, int chunk_begin,
+                          int chunk_end, int causal, int own_chunk_only, float scale,
+                          const int32_t* slab_pairs, int num_slab_pairs, int softmax, int zero_rows_from,
+                          int window_row0, int window_rows, const double* tau_per_head, uint8_t* mask,
+                          int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int keep_sink,
+                          int keep_recent, int stages, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Block-sparse FlashAttention forward.  Replaces the call
  *   block_sparse_attn_func(q, k, v, cu_q, cu_k, head_mask_type, None, mask,
  *                          q_len, k_len, p_dropout=0, deterministic=True,

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void mfma_rate_probe_kernel(const probe_bf16x8
 }
 }  // namespace xattn
 
-extern "C" int xattn_abi_version(void) { return 6; }
+extern "C" int xattn_abi_version(void) { return 7; }
 
 extern "C" const char* xattn_error_string(int code) {
   switch (code) {

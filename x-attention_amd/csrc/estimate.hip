@@ -22,7 +22,7 @@
 //    and adds the block_size/S rows of each query block.
 #include <mutex>
 
-#include "xattn_common.h"
+#include "select_row.h"
 #include "xattn_hip.h"
 
 namespace xattn {
@@ -390,6 +390,39 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   wait_vm0();   // the repeats the last tile issued into LDS
 }
 
+// The arithmetic of the normalisation, shared by the stand-alone pass and the fused normalise-and-select kernel
+// so that both give the same bits (fixed operation order, no contraction into fused multiply-adds).
+#pragma clang fp contract(off)
+// folds tile T's maximum / sum into a running (M, L)
+__device__ __forceinline__ void stat_step(float& M, float& L, float mt, float lt) {
+  const float Mn = fmaxf(M, mt);
+  const float safe = (Mn == -INFINITY) ? 0.f : Mn;
+  L = L * fast_exp2(M - safe) + lt * fast_exp2(mt - safe);
+  M = Mn;
+}
+// combines the four partial (M, L) of a row (tiles T = first + w, + 4, ... for w = 0..3) into the row's
+// maximum (0 when the row sees nothing, or without softmax) and 1 / sum (0 for rows that give zeros)
+__device__ __forceinline__ void stat_combine(const float (&Mw)[4], const float (&Lw)[4], bool real_row, int no_softmax,
+                                             float* rowM, float* rowInv) {
+  const float Mr = fmaxf(fmaxf(Mw[0], Mw[1]), fmaxf(Mw[2], Mw[3]));
+  const float safe = (Mr == -INFINITY) ? 0.f : Mr;
+  float Lr = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) Lr += Lw[w] * fast_exp2(Mw[w] - safe);
+  const bool real = real_row && Lr > 0.f;
+  // without softmax the partial sums are referred to 2^0 and left unnormalised
+  *rowM = no_softmax ? 0.f : safe;
+  *rowInv = real ? (no_softmax ? 1.f : 1.f / Lr) : 0.f;
+}
+// normalised partial sums of four consecutive rows, added up
+__device__ __forceinline__ float group_sum4(const f32x4& pv, const f32x4& mt, const f32x4& rM, const f32x4& rI) {
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc += (rI[i] != 0.f) ? pv[i] * (fast_exp2(mt[i] - rM[i]) * rI[i]) : 0.f;
+  return acc;
+}
+#pragma clang fp contract(fast)
+
 // One workgroup = 64 consecutive reshaped query rows of one head.
 // Pass 1 (lane <-> row, wavefronts split the 128-key tiles) combines the tile
 // maxima / sums into each row's softmax statistics.  Pass 2 rescales the partial
@@ -418,27 +451,15 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
     int hi = row_hi(p, mc);
     hi = hi < p.n_rk - 1 ? hi : p.n_rk - 1;
     float M = -INFINITY, L = 0.f;
-    for (int T = lo / kSub + wave; T <= hi / kSub; T += 4) {
-      const float mt = Mst[(int64_t)T * p.rows + mrel];
-      const float lt = Lst[(int64_t)T * p.rows + mrel];
-      const float Mn = fmaxf(M, mt);
-      const float safe = (Mn == -INFINITY) ? 0.f : Mn;
-      L = L * fast_exp2(M - safe) + lt * fast_exp2(mt - safe);
-      M = Mn;
-    }
+    for (int T = lo / kSub + wave; T <= hi / kSub; T += 4)
+      stat_step(M, L, Mst[(int64_t)T * p.rows + mrel], Lst[(int64_t)T * p.rows + mrel]);
     redM[wave][lane] = M;
     redL[wave][lane] = L;
     __syncthreads();
     if (wave == 0) {
-      const float Mr = fmaxf(fmaxf(redM[0][lane], redM[1][lane]), fmaxf(redM[2][lane], redM[3][lane]));
-      const float safe = (Mr == -INFINITY) ? 0.f : Mr;
-      float Lr = 0.f;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) Lr += redL[w][lane] * fast_exp2(redM[w][lane] - safe);
-      const bool real = row_ok && mc < p.real_rows && Lr > 0.f;
-      // without softmax the partial sums are referred to 2^0 and left unnormalised
-      rowM[lane] = p.no_softmax ? 0.f : safe;
-      rowInv[lane] = real ? (p.no_softmax ? 1.f : 1.f / Lr) : 0.f;
+      const float Mw[4] = {redM[0][lane], redM[1][lane], redM[2][lane], redM[3][lane]};
+      const float Lw[4] = {redL[0][lane], redL[1][lane], redL[2][lane], redL[3][lane]};
+      stat_combine(Mw, Lw, row_ok && mc < p.real_rows, p.no_softmax, &rowM[lane], &rowInv[lane]);
     }
     __syncthreads();
   }
@@ -478,14 +499,136 @@ __global__ __launch_bounds__(256) void estimate_normalize_kernel(EstParams p) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int kb = kb0 + 16 * u + kgrp;
-      float acc = 0.f;
-      if (live[u]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc += (rI[i] != 0.f) ? pv[u][i] * (fast_exp2(mt[u][i] - rM[i]) * rI[i]) : 0.f;
-      }
+      float acc = live[u] ? group_sum4(pv[u], mt[u], rM, rI) : 0.f;
 #pragma unroll
       for (int d = 1; d < kLanesPerBlock; d <<= 1) acc += __shfl_xor(acc, d, 64);
       if (rows_ok && kb < p.nkb && (l16 % kLanesPerBlock) == 0) out[kb] = acc;
+    }
+  }
+}
+
+// Normalisation and selection in one pass, for callers that want the column lists (or the mask) and not the
+// block sums: a workgroup of QB wavefronts takes QB consecutive q-block rows of one head (QB * RBS reshaped
+// query rows), computes their softmax statistics and normalised block sums exactly as the kernel above does -
+// same loads, same operation order - but leaves the sums in LDS, where wavefront i then runs the selection of
+// row i (select_row.h).  The block sums never travel to memory and back.
+template <int RBS>
+__global__ __launch_bounds__(256) void estimate_select_kernel(EstParams p, SelParams sp, int qb_per_wg) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rows_wg = qb_per_wg * RBS;                   // reshaped rows of the workgroup (<= 128)
+  const int nkb_pad = (p.nkb + 15) & ~15;
+  // LDS: statistics, then per wavefront its sort keys (with the row's block sums) and flags
+  float* redM = reinterpret_cast<float*>(smem);          // [4][rows_wg]
+  float* redL = redM + 4 * rows_wg;                      // [4][rows_wg]
+  float* rowM = redL + 4 * rows_wg;                      // [rows_wg]
+  float* rowInv = rowM + rows_wg;                        // [rows_wg]
+  char* per_wave = smem + 10 * rows_wg * sizeof(float);
+  // per wavefront: sort keys, flags; the row's block sums share the tail of the key array (select_row.h)
+  const size_t wave_bytes = (size_t)sp.npow2 * 8 + nkb_pad;
+  const size_t xs_off = (size_t)sp.npow2 * 8 - (size_t)nkb_pad * 4;
+
+  const int qrows = (p.row_end - p.row_begin) / RBS;     // q-block rows of this call
+  const int groups = (qrows + qb_per_wg - 1) / qb_per_wg;
+  const int head = blockIdx.x / groups;
+  const int grp = blockIdx.x % groups;
+  const int strip0 = p.row_begin + grp * rows_wg;        // first reshaped row of the workgroup
+  const float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
+  const float* Mst = p.Mt + (int64_t)head * p.nT * p.rows;
+  const float* Lst = p.Lt + (int64_t)head * p.nT * p.rows;
+
+  // pass 1: thread (row, w) folds tiles first + w, + 4, ... of its row
+  for (int idx = tid; idx < rows_wg * 4; idx += blockDim.x) {
+    const int lrow = idx % rows_wg, w = idx / rows_wg;
+    const int m = strip0 + lrow;
+    const int mc = m < p.row_end ? m : p.row_end - 1;
+    const int mrel = mc - p.row_begin;
+    const int lo = row_lo(p, mc);
+    int hi = row_hi(p, mc);
+    hi = hi < p.n_rk - 1 ? hi : p.n_rk - 1;
+    float M = -INFINITY, L = 0.f;
+    // eight tiles' statistics are requested before the first is folded in (the folding is a dependent chain)
+    for (int T0 = lo / kSub + w; T0 <= hi / kSub; T0 += 32) {
+      float mt[8], lt[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int T = T0 + 4 * u;
+        if (T <= hi / kSub) {
+          mt[u] = Mst[(int64_t)T * p.rows + mrel];
+          lt[u] = Lst[(int64_t)T * p.rows + mrel];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (T0 + 4 * u <= hi / kSub) stat_step(M, L, mt[u], lt[u]);
+    }
+    redM[w * rows_wg + lrow] = M;
+    redL[w * rows_wg + lrow] = L;
+  }
+  __syncthreads();
+  for (int lrow = tid; lrow < rows_wg; lrow += blockDim.x) {
+    const int m = strip0 + lrow;
+    const bool row_ok = m < p.row_end;
+    const float Mw[4] = {redM[lrow], redM[rows_wg + lrow], redM[2 * rows_wg + lrow], redM[3 * rows_wg + lrow]};
+    const float Lw[4] = {redL[lrow], redL[rows_wg + lrow], redL[2 * rows_wg + lrow], redL[3 * rows_wg + lrow]};
+    stat_combine(Mw, Lw, row_ok && m < p.real_rows, p.no_softmax, &rowM[lrow], &rowInv[lrow]);
+  }
+  __syncthreads();
+
+  // pass 2: a thread owns 4 consecutive rows; lpk threads cover the workgroup's rows, the rest of the
+  // thread index runs over key blocks
+  {
+    constexpr int kLanesPerBlock = RBS / 4;
+    const int lpk = rows_wg / 4;
+    const int l = tid % lpk, kgrp = tid / lpk, kb_step = blockDim.x / lpk;
+    const int m4 = strip0 + l * 4;
+    const bool rows_ok = m4 < p.row_end;
+    const int mc4 = rows_ok ? m4 : p.row_begin;
+    const int mrel4 = mc4 - p.row_begin;
+    const f32x4 rM = *reinterpret_cast<const f32x4*>(rowM + l * 4);
+    const f32x4 rI = *reinterpret_cast<const f32x4*>(rowInv + l * 4);
+    const int kb_lo = row_lo(p, mc4) / RBS;
+    int hi4 = row_hi(p, mc4);
+    hi4 = hi4 < p.n_rk - 1 ? hi4 : p.n_rk - 1;
+    const int kb_hi = hi4 / RBS;
+    float* xs = reinterpret_cast<float*>(per_wave + (size_t)(l / kLanesPerBlock) * wave_bytes + xs_off);
+    float* gout = p.sums ? p.sums + ((int64_t)head * p.win_rows + (mc4 / RBS - p.win_row0)) * p.nkb : nullptr;
+    constexpr int kUnroll = 8;
+    for (int kb0 = kgrp; kb0 < p.nkb; kb0 += kb_step * kUnroll) {
+      f32x4 pv[kUnroll], mt[kUnroll];
+      bool live[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int kb = kb0 + kb_step * u;
+        live[u] = rows_ok && kb < p.nkb && kb >= kb_lo && kb <= kb_hi;
+        if (live[u]) {
+          const int T = (kb * RBS) / kSub;
+          mt[u] = *reinterpret_cast<const f32x4*>(Mst + (int64_t)T * p.rows + mrel4);
+          pv[u] = *reinterpret_cast<const f32x4*>(Pst + (int64_t)kb * p.rows + mrel4);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int kb = kb0 + kb_step * u;
+        float acc = live[u] ? group_sum4(pv[u], mt[u], rM, rI) : 0.f;
+#pragma unroll
+        for (int d = 1; d < kLanesPerBlock; d <<= 1) acc += __shfl_xor(acc, d, 64);
+        if (kb < p.nkb && (l % kLanesPerBlock) == 0) {
+          xs[kb] = acc;
+          if (gout && rows_ok) gout[kb] = acc;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // selection: wavefront i takes q-block row i of the group
+  if (wave < qb_per_wg) {
+    const int row = strip0 / RBS + wave;                 // q-block row (row_begin is a multiple of RBS)
+    if (row < p.row_end / RBS) {
+      char* mine = per_wave + (size_t)wave * wave_bytes;
+      select_row(sp, reinterpret_cast<const float*>(mine + xs_off), head, row, reinterpret_cast<uint64_t*>(mine),
+                 reinterpret_cast<uint8_t*>(mine + (size_t)sp.npow2 * 8), lane);
     }
   }
 }
@@ -619,16 +762,34 @@ extern "C" size_t xattn_estimate_workspace_bytes(int num_heads, int q_len, int k
   return workspace_bytes(num_heads, g, c * g.rcs);   // (an upper bound when query rows are subsampled)
 }
 
-extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, void* workspace,
-                                         size_t workspace_size, float* scores_out, int num_heads,
-                                         int num_kv_heads, int q_len, int k_len, int head_dim,
-                                         int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
-                                         int64_t k_stride_n, int stride, int block_size, int chunk_size,
-                                         int chunk_begin, int chunk_end, int causal, int own_chunk_only,
-                                         float scale, const int32_t* slab_pairs, int num_slab_pairs,
-                                         int softmax, int kdb, int zero_rows_from, int window_row0,
-                                         int window_rows, void* stream) {
-  if (!q || !k || !block_sums || !workspace) return XATTN_ERR_NULL;
+namespace {
+// what the fused normalise-and-select pass needs beside the estimator's own arguments
+struct SelectArgs {
+  const double* tau;
+  uint8_t* mask;
+  int32_t* col_idx;
+  int32_t* col_cnt;
+  int64_t idx_pitch;
+  int keep_sink, keep_recent;
+  int stages;               // bit 0: run the GEMM pass, bit 1: run the normalise-and-select pass
+};
+
+int estimate_impl(const void* q, const void* k, float* block_sums, void* workspace, size_t workspace_size,
+                  float* scores_out, int num_heads, int num_kv_heads, int q_len, int k_len, int head_dim,
+                  int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h, int64_t k_stride_n, int stride,
+                  int block_size, int chunk_size, int chunk_begin, int chunk_end, int causal, int own_chunk_only,
+                  float scale, const int32_t* slab_pairs, int num_slab_pairs, int softmax, int kdb,
+                  int zero_rows_from, int window_row0, int window_rows, void* stream, const SelectArgs* sel) {
+  if (!q || !k || !workspace) return XATTN_ERR_NULL;
+  if (!block_sums && !sel) return XATTN_ERR_NULL;
+  if (sel) {
+    if (!sel->tau) return XATTN_ERR_NULL;
+    if ((sel->col_idx == nullptr) != (sel->col_cnt == nullptr)) return XATTN_ERR_NULL;
+    if (!sel->mask && !sel->col_idx) return XATTN_ERR_NULL;     // nothing to write
+    if (sel->col_idx && sel->idx_pitch < 1) return XATTN_ERR_SHAPE;
+    if (kdb != 1) return XATTN_ERR_SHAPE;                        // the fused pass needs whole query blocks of rows
+    if (!(sel->stages & 3) || (sel->stages & ~3)) return XATTN_ERR_SHAPE;
+  }
   if (head_dim != kHeadDim) return XATTN_ERR_HEAD_DIM;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return XATTN_ERR_HEADS;
   if (block_size != 128 || (stride != 4 && stride != 8 && stride != 16)) return XATTN_ERR_STRIDE;
@@ -712,19 +873,61 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
   const dim3 grid2((p.rows + 63) / 64, num_heads);
   if (grid2.y > 65535) return XATTN_ERR_SHAPE;
   const size_t lds = 2 * (size_t)kStageBytes;
+  // the fused normalise-and-select pass: QB q-block rows (one wavefront each) per workgroup, as many as keep a
+  // workgroup's LDS (statistics + per wavefront: the row's sums, sort keys, flags) within 64 KiB
+  SelParams sp;
+  int qb_per_wg = 0;
+  size_t lds_sel = 0;
+  dim3 grid_sel(1);
+  if (sel) {
+    if (g.nkb > 8192) return XATTN_ERR_SHAPE;      // (longer rows: block sums through memory, xattn_select_blocks)
+    const int bpc = chunk_size / block_size;
+    sp.sums = nullptr; sp.tau = sel->tau; sp.mask = sel->mask; sp.col_idx = sel->col_idx; sp.col_cnt = sel->col_cnt;
+    sp.idx_pitch = sel->idx_pitch; sp.H = num_heads; sp.nqb = g.nqb; sp.nkb = g.nkb;
+    sp.row_begin = chunk_begin * bpc; sp.row_end = chunk_end * bpc; sp.diag_offset = g.nkb - g.nqb;
+    sp.win_row0 = p.win_row0; sp.win_rows = p.win_rows;
+    sp.causal = p.causal; sp.keep_sink = sel->keep_sink ? 1 : 0; sp.keep_recent = sel->keep_recent ? 1 : 0;
+    sp.list_cols = (k_len + block_size - 1) / block_size; sp.q_len = q_len; sp.kv_off = k_len - q_len;
+    sp.blocks_per_chunk = bpc;
+    int np2 = 64;
+    while (np2 < g.nkb) np2 <<= 1;
+    sp.npow2 = np2;
+    const size_t nkb_pad = ((size_t)g.nkb + 15) & ~(size_t)15;
+    const size_t wave_bytes = (size_t)np2 * 8 + nkb_pad;
+    qb_per_wg = 4;
+    while (qb_per_wg > 1 && (qb_per_wg * (wave_bytes + 10 * p.rbs * sizeof(float)) > 64 * 1024 || qb_per_wg * p.rbs > 128))
+      qb_per_wg >>= 1;
+    lds_sel = qb_per_wg * (wave_bytes + 10 * p.rbs * sizeof(float));
+    const int qrows = p.rows / p.rbs;
+    const int64_t wgs = (int64_t)num_heads * ((qrows + qb_per_wg - 1) / qb_per_wg);
+    if (wgs > 0x7fffffff) return XATTN_ERR_SHAPE;
+    grid_sel = dim3((unsigned)wgs);
+  }
+  auto launch_rest = [&](auto normalize, auto fused) -> hipError_t {
+    if (!sel) {
+      if (kdb == 1) hipLaunchKernelGGL(normalize, grid2, dim3(256), 0, s, p);
+      return hipSuccess;
+    }
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(fused), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)lds_sel);
+    if (e2 != hipSuccess) return e2;
+    hipLaunchKernelGGL(fused, grid_sel, dim3(64 * qb_per_wg), lds_sel, s, p, sp, qb_per_wg);
+    return hipSuccess;
+  };
+  const bool run_gemm = !sel || (sel->stages & 1), run_rest = !sel || (sel->stages & 2);
   hipError_t e = hipSuccess;
   switch (p.rbs) {
     case 8:
-      e = launch_gemm<8>(p, grid1, lds, s);
-      if (e == hipSuccess && kdb == 1) hipLaunchKernelGGL(estimate_normalize_kernel<8>, grid2, dim3(256), 0, s, p);
+      if (run_gemm) e = launch_gemm<8>(p, grid1, lds, s);
+      if (e == hipSuccess && run_rest) e = launch_rest(&estimate_normalize_kernel<8>, &estimate_select_kernel<8>);
       break;
     case 16:
-      e = launch_gemm<16>(p, grid1, lds, s);
-      if (e == hipSuccess && kdb == 1) hipLaunchKernelGGL(estimate_normalize_kernel<16>, grid2, dim3(256), 0, s, p);
+      if (run_gemm) e = launch_gemm<16>(p, grid1, lds, s);
+      if (e == hipSuccess && run_rest) e = launch_rest(&estimate_normalize_kernel<16>, &estimate_select_kernel<16>);
       break;
     default:
-      e = launch_gemm<32>(p, grid1, lds, s);
-      if (e == hipSuccess && kdb == 1) hipLaunchKernelGGL(estimate_normalize_kernel<32>, grid2, dim3(256), 0, s, p);
+      if (run_gemm) e = launch_gemm<32>(p, grid1, lds, s);
+      if (e == hipSuccess && run_rest) e = launch_rest(&estimate_normalize_kernel<32>, &estimate_select_kernel<32>);
       break;
   }
   if (e != hipSuccess) return XATTN_ERR_LAUNCH;
@@ -733,4 +936,37 @@ extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* bl
     hipLaunchKernelGGL(estimate_normalize_rows_kernel, grid3, dim3(256), 0, s, p);
   }
   return hipGetLastError() == hipSuccess ? XATTN_OK : XATTN_ERR_LAUNCH;
+}
+}  // namespace
+
+extern "C" int xattn_estimate_block_sums(const void* q, const void* k, float* block_sums, void* workspace,
+                                         size_t workspace_size, float* scores_out, int num_heads,
+                                         int num_kv_heads, int q_len, int k_len, int head_dim,
+                                         int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
+                                         int64_t k_stride_n, int stride, int block_size, int chunk_size,
+                                         int chunk_begin, int chunk_end, int causal, int own_chunk_only,
+                                         float scale, const int32_t* slab_pairs, int num_slab_pairs,
+                                         int softmax, int kdb, int zero_rows_from, int window_row0,
+                                         int window_rows, void* stream) {
+  if (!block_sums) return XATTN_ERR_NULL;
+  return estimate_impl(q, k, block_sums, workspace, workspace_size, scores_out, num_heads, num_kv_heads, q_len, k_len,
+                       head_dim, q_stride_h, q_stride_n, k_stride_h, k_stride_n, stride, block_size, chunk_size,
+                       chunk_begin, chunk_end, causal, own_chunk_only, scale, slab_pairs, num_slab_pairs, softmax, kdb,
+                       zero_rows_from, window_row0, window_rows, stream, nullptr);
+}
+
+extern "C" int xattn_estimate_select(const void* q, const void* k, float* block_sums, void* workspace,
+                                     size_t workspace_size, int num_heads, int num_kv_heads, int q_len, int k_len,
+                                     int head_dim, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_h,
+                                     int64_t k_stride_n, int stride, int block_size, int chunk_size, int chunk_begin,
+                                     int chunk_end, int causal, int own_chunk_only, float scale,
+                                     const int32_t* slab_pairs, int num_slab_pairs, int softmax, int zero_rows_from,
+                                     int window_row0, int window_rows, const double* tau_per_head, uint8_t* mask,
+                                     int32_t* col_idx, int32_t* col_cnt, int64_t idx_pitch, int keep_sink,
+                                     int keep_recent, int stages, void* stream) {
+  const SelectArgs sel = {tau_per_head, mask, col_idx, col_cnt, idx_pitch, keep_sink, keep_recent, stages};
+  return estimate_impl(q, k, block_sums, workspace, workspace_size, nullptr, num_heads, num_kv_heads, q_len, k_len,
+                       head_dim, q_stride_h, q_stride_n, k_stride_h, k_stride_n, stride, block_size, chunk_size,
+                       chunk_begin, chunk_end, causal, own_chunk_only, scale, slab_pairs, num_slab_pairs, softmax, 1,
+                       zero_rows_from, window_row0, window_rows, stream, &sel);
 }

@@ -103,7 +103,7 @@ class _Plan:
 
     def __init__(self, query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
                  keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs=None, softmax=True, kdb=1,
-                 want_mask=True, group_limit=None):
+                 want_mask=True, group_limit=None, want_sums=True):
         self.lib = _hb.lib()
         self.kdb = int(kdb)
         self.softmax = bool(softmax)
@@ -173,7 +173,11 @@ class _Plan:
         # Block sums, mask and column lists hold a window of q-block rows: all of them, or - when a byte
         # limit is given and they would exceed it - one group of whole query chunks at a time, which the
         # caller works through with window(); the buffers are reused from group to group.
-        per_row = self.heads * (self.nkb * 4 + (self.nkb if want_mask else 0)
+        # Without the block sums (the operator never looks at them) normalisation and selection run as one
+        # pass that keeps them in LDS; rows of more than 8192 key blocks and subsampled query rows go
+        # through memory (xattn_estimate_select's limits).
+        self.fused = (not want_sums) and (not dump_scores) and self.kdb == 1 and self.nkb <= 8192
+        per_row = self.heads * ((0 if self.fused else self.nkb * 4) + (self.nkb if want_mask else 0)
                                 + ((self.list_cols + 1) * 4 if want_lists else 0))
         self.chunks_per_group = self.q_chunks
         if group_limit is not None and per_row * self.nqb > group_limit:
@@ -182,7 +186,9 @@ class _Plan:
         self.win_row0 = 0
         with torch.cuda.device(dev):
             self.workspace = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
-            self.sums = torch.empty((self.heads, self.win_rows, self.nkb), dtype=torch.float32, device=dev)
+            self.sums = None
+            if not self.fused:
+                self.sums = torch.empty((self.heads, self.win_rows, self.nkb), dtype=torch.float32, device=dev)
             self.scores = None
             if dump_scores:
                 self.scores = torch.zeros(
@@ -225,6 +231,38 @@ class _Plan:
             "xattn_estimate_block_sums",
         )
 
+    def estimate_select(self, chunk_begin, chunk_end, stream, stages=3):
+        """Estimator and selection of query chunks [chunk_begin, chunk_end) without block sums in memory
+        (``self.fused`` plans only).  ``stages``: 1 = the MFMA pass, 2 = normalise and select, 3 = both."""
+        if chunk_end - chunk_begin > self.chunks_per_call:
+            for c in range(chunk_begin, chunk_end, self.chunks_per_call):
+                self.estimate_select(c, min(chunk_end, c + self.chunks_per_call), stream, stages)
+            return
+        q, k = self.q, self.k
+        lists = self.col_idx is not None
+        _hb.check(
+            self.lib.xattn_estimate_select(
+                q.data_ptr(), k.data_ptr(), None, self.workspace.data_ptr(), self.ws_bytes,
+                self.heads, self.kv_heads, self.q_len, self.k_len, 128,
+                q.stride(1), q.stride(2), k.stride(1), k.stride(2),
+                self.stride, self.block_size, self.chunk_size, chunk_begin, chunk_end,
+                int(self.causal), int(self.own_chunk_only), self.scale, self.pairs, self.n_pairs,
+                int(self.softmax), self.zero_rows_from, self.win_row0, self.win_rows,
+                self.tau.data_ptr(), self.mask.data_ptr() if self.mask is not None else None,
+                self.col_idx.data_ptr() if lists else None, self.col_cnt.data_ptr() if lists else None,
+                self.list_cols, int(self.keep_sink), int(self.keep_recent), stages, stream,
+            ),
+            "xattn_estimate_select",
+        )
+
+    def run(self, chunk_begin, chunk_end, stream):
+        """Estimate and selection of query chunks [chunk_begin, chunk_end), by whichever path the plan uses."""
+        if self.fused:
+            self.estimate_select(chunk_begin, chunk_end, stream)
+        else:
+            self.estimate(chunk_begin, chunk_end, stream)
+            self.select(chunk_begin * self.blocks_per_chunk, chunk_end * self.blocks_per_chunk, stream)
+
     def select(self, row_begin, row_end, stream):
         lists = self.col_idx is not None
         _hb.check(
@@ -263,6 +301,7 @@ def estimate_and_select(
     softmax=True,
     kdb=1,
     want_mask=True,
+    want_sums=True,
 ):
     """Runs the estimator and selection kernels over all query chunks, one launch each.
 
@@ -271,19 +310,36 @@ def estimate_and_select(
     [H, Nq_p] for :func:`block_sparse_attention` (``want_mask=False`` skips the
     byte mask, which the attention kernel does not read).
 
+    ``want_sums=False`` (what the operator asks for) leaves ``sums`` out of the
+    result: normalisation and selection then run as one pass that keeps the block
+    sums in LDS (``xattn_estimate_select``); lists and mask are the same.
+
     ``marks``, when a list, receives ``(label, torch.cuda.Event)`` pairs recorded
-    on the current stream before the estimator, between estimator and selection
-    and after selection (for per-kernel timing).
+    on the current stream before the estimator, between its MFMA pass and what
+    follows (normalisation + selection, or - with block sums - between
+    estimator and selection) and after selection (for per-kernel timing).
     """
     plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
                  keep_sink, keep_recent, block_size, want_lists, dump_scores, slab_pairs, softmax, kdb,
-                 want_mask=want_mask)
+                 want_mask=want_mask, want_sums=want_sums)
     with torch.cuda.device(plan.dev):
         stream = _stream_ptr(plan.dev)
         _mark(marks, "estimate_begin")
-        plan.estimate(0, plan.q_chunks, stream)
-        _mark(marks, "select_begin")
-        plan.select(0, plan.nqb, stream)
+        if plan.fused and marks is None:
+            plan.estimate_select(0, plan.q_chunks, stream)
+        elif plan.fused:
+            # the two passes as separate calls, so that an event can sit between them
+            for c in range(0, plan.q_chunks, plan.chunks_per_call):
+                plan.estimate_select(c, min(plan.q_chunks, c + plan.chunks_per_call), stream, stages=1)
+                if c == 0 and plan.chunks_per_call >= plan.q_chunks:
+                    _mark(marks, "select_begin")
+                plan.estimate_select(c, min(plan.q_chunks, c + plan.chunks_per_call), stream, stages=2)
+            if plan.chunks_per_call < plan.q_chunks:
+                _mark(marks, "select_begin")
+        else:
+            plan.estimate(0, plan.q_chunks, stream)
+            _mark(marks, "select_begin")
+            plan.select(0, plan.nqb, stream)
         _mark(marks, "select_end")
     return plan.result()
 
@@ -420,7 +476,8 @@ def Xattention_prefill(
     # (128k tokens: 0.26 GB); longer sequences go through the three stages one group of query chunks at a
     # time on buffers of one group, so the extra memory stays bounded however long the sequence is.
     plan = _Plan(query_states, key_states, stride, threshold, chunk_size, causal, norm, use_triton,
-                 keep_sink, keep_recent, block_size, True, False, kdb=kdb, want_mask=False, group_limit=GROUP_LIMIT)
+                 keep_sink, keep_recent, block_size, True, False, kdb=kdb, want_mask=False, group_limit=GROUP_LIMIT,
+                 want_sums=False)
     dev = plan.dev
     v = _check_qk(value_states, "value_states")
     nb = (plan.q_len + block_size - 1) // block_size
@@ -430,8 +487,7 @@ def Xattention_prefill(
         bpc = plan.blocks_per_chunk
         for c0, c1 in plan.groups():
             plan.window(c0)
-            plan.estimate(c0, c1, stream)
-            plan.select(c0 * bpc, c1 * bpc, stream)
+            plan.run(c0, c1, stream)
             qb0, qb1 = c0 * bpc, min(nb, c1 * bpc)
             if qb0 < qb1:
                 block_sparse_attention(plan.q, plan.k, v, plan.col_idx, plan.col_cnt, causal=causal, out=out,

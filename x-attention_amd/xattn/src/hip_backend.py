@@ -21,6 +21,12 @@ _SIGNATURES = {
         [c_vp, c_vp, c_vp, c_vp, c_sz, c_vp] + [c_i32] * 5 + [c_i64] * 4 + [c_i32] * 7
         + [c_f32, ctypes.POINTER(c_i32), c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp],
     ),
+    "xattn_estimate_select": (
+        c_i32,
+        [c_vp, c_vp, c_vp, c_vp, c_sz] + [c_i32] * 5 + [c_i64] * 4 + [c_i32] * 7
+        + [c_f32, ctypes.POINTER(c_i32), c_i32, c_i32, c_i32, c_i32, c_i32]
+        + [c_vp] * 4 + [c_i64, c_i32, c_i32, c_i32, c_vp],
+    ),
     "xattn_select_blocks": (
         c_i32,
         [c_vp] * 5 + [c_i64] + [c_i32] * 15 + [c_vp],
