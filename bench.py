@@ -7,12 +7,21 @@ A step is one pass of the hot path - antidiagonal estimate, block selection,
 block-sparse attention - over one synthetic single-layer workload whose q/k/v
 already sit in HBM.  The default workload is the headline one (L=131072,
 32 query / 8 KV heads, d=128, stride 16, tau 0.9, chunk 16384, causal, bf16).
-Prints ONE JSON line: the per-layer time (estimate + sparse), the speedup over
-this library's own dense causal FlashAttention, the roofline of the dominant
-kernel (block-sparse attention, bf16 MFMA, flops of the computed blocks) and a
-CPU baseline (the torch restatement of the reference path on workload 0).
+Prints ONE JSON line: the per-layer time (estimate + select + sparse attention;
+mean, median and minimum over the timed steps), the speedup over this
+library's own dense FlashAttention, the roofline of the longer of the two MFMA
+kernels (the estimator's GEMM at the headline) and of the other one, the same
+measurements for the other GPU workloads, two library yardsticks (a bf16 GEMM
+of the estimator's shape, a causal flash attention) and a CPU baseline (the
+torch restatement of the reference path on workload 0).
+
+Timing protocol (the reference's eval/efficiency/attention_speedup.py:82-132
+uses 30 warm-ups and 50 timed runs): W untimed warm-up steps, then K timed steps
+with HIP events on the launch stream between the stages of every step; the dense
+baseline gets its own warm-ups and timed launches.
 """
 import argparse
+import hashlib
 import json
 import os
 import statistics
@@ -30,24 +39,47 @@ PEAK_HBM_GBS = 8000.0
 # this process): the summary of those runs for the headline workload is kept as a table under profiles/ and read here.
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "bench_headline_hbm_traffic.md")
 HEADLINE = "cfg2_llama8b_L131072_gqa32x8_S16"
+KERNEL_SOURCES = ("attn_tiles.h", "block_sparse_attn.hip", "estimate.hip", "select_row.h", "select_blocks.hip",
+                  "xattn_common.h")
+
+
+def kernel_source_hash():
+    """sha256 (16 hex digits) over the sources of the measured kernels.  The counter summary under profiles/
+    names the hash it was taken at; a summary taken at other sources is not quoted."""
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "x-attention_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def measured_traffic_bytes(kernel_prefix):
     """Scaled total bytes of the first table row of the traffic summary whose kernel name starts with
-    ``kernel_prefix`` (last column, in GB), or None when the summary or the row is missing."""
+    ``kernel_prefix`` (last column, in GB); None when the summary or the row is missing, or when the summary
+    was taken at other kernel sources than the ones in the tree."""
     try:
         with open(TRAFFIC_SUMMARY) as f:
-            for line in f:
-                cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
-                if len(cells) >= 6 and cells[0].startswith(kernel_prefix):
-                    return float(cells[-1]) * 1e9
-    except (OSError, ValueError):
-        pass
+            text = f.read()
+    except OSError:
+        return None
+    if ("kernel sources sha256/16: " + kernel_source_hash()) not in text:
+        return None
+    for line in text.splitlines():
+        cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 6 and cells[0].startswith(kernel_prefix):
+            try:
+                return float(cells[-1]) * 1e9
+            except ValueError:
+                return None
     return None
 
 
 def _ms(a, b):
     return a.elapsed_time(b)
+
+
+def _stats(xs):
+    return {"mean": round(statistics.mean(xs), 4), "median": round(statistics.median(xs), 4), "min": round(min(xs), 4)}
 
 
 def cpu_baseline(reps=5, warmup=2):
@@ -180,60 +212,245 @@ def mfma_probe(dev):
     return res
 
 
+def flops_and_bytes(w, L, chunk, n_sel):
+    """Algorithmic work of the three stages for a workload of length L."""
+    H = w.heads
+    nb = (L + 127) // 128
+    Lp = (L + chunk - 1) // chunk * chunk
+    n_r = Lp // w.stride
+    nkb_p = Lp // 128
+    rbs = 128 // w.stride
+    causal = w.causal
+    full_blocks = H * nb * (nb + 1) // 2 if causal else H * nb * nb
+    f_est = (2.0 * w.stride * 128 * H * n_r * (n_r + 1) / 2) if causal else (2.0 * w.stride * 128 * H * n_r * n_r)
+    f_dense = (4.0 * 128 * H * L * (L + 1) / 2) if causal else (4.0 * 128 * H * L * L)
+    f_sparse = 4.0 * 128 ** 3 * n_sel
+    # what the normalise-and-select pass moves: the visible part of the partial block sums (fp32 [H][Nk_p][n_r])
+    # and of the tile statistics (two fp32 [H][n_r/128][n_r]) in, the column lists and counts out
+    vis = 0.5 if causal else 1.0
+    pass_bytes = 4.0 * H * n_r * nkb_p * vis + 2 * 4.0 * H * n_r * (n_r / 128.0) * vis + 4.0 * (n_sel + H * nkb_p)
+    # the selection as the reference stages it: the full block-sum matrix in, a byte mask and the lists out
+    survey_bytes = H * nkb_p * nkb_p * 5 + 4.0 * (n_sel + H * nkb_p)
+    return dict(full_blocks=full_blocks, f_est=f_est, f_dense=f_dense, f_sparse=f_sparse, pass_bytes=pass_bytes,
+                survey_bytes=survey_bytes, rbs=rbs)
+
+
+def measure(w, q, k, v, L, tau, chunk, steps, warmup, dense_steps, dense_warmup):
+    """Times `steps` passes of estimate -> select -> sparse attention (what the operator runs: column lists only,
+    block sums kept in LDS) after `warmup` untimed ones, and the dense baseline.  Returns per-stage statistics."""
+    import torch
+    from xattn.src.Xattention import block_sparse_attention, estimate_and_select
+
+    def step(marks):
+        r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, marks=marks, want_mask=False,
+                                want_sums=False)
+        out = block_sparse_attention(q, k, v, r["col_idx"], r["col_cnt"], causal=w.causal)
+        if marks is not None:
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            marks.append(("sparse_end", ev))
+        return r, out
+
+    with torch.no_grad():
+        for _ in range(warmup):
+            r, out = step(None)
+        torch.cuda.synchronize()
+        all_marks = []
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            m = []
+            r, out = step(m)
+            all_marks.append(dict(m))
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        est = [_ms(m["estimate_begin"], m["select_begin"]) for m in all_marks]
+        sel = [_ms(m["select_begin"], m["select_end"]) for m in all_marks]
+        att = [_ms(m["select_end"], m["sparse_end"]) for m in all_marks]
+        tot = [_ms(m["estimate_begin"], m["sparse_end"]) for m in all_marks]
+        del out
+        # dense FlashAttention written the same way (same kernel, every visible block)
+        for _ in range(dense_warmup):
+            block_sparse_attention(q, k, v, causal=w.causal)
+        torch.cuda.synchronize()
+        dense = []
+        for _ in range(dense_steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            block_sparse_attention(q, k, v, causal=w.causal)
+            e1.record()
+            torch.cuda.synchronize()
+            dense.append(_ms(e0, e1))
+    nb = (L + 127) // 128
+    n_sel = int(r["col_cnt"][:, :nb].sum().item())
+    return dict(est=est, sel=sel, att=att, tot=tot, dense=dense, wall_ms=wall_ms, n_sel=n_sel, col_cnt=r["col_cnt"])
+
+
+def mask_parity(w, q, k, tau, chunk, col_cnt):
+    """Block-mask parity with the oracle (fp32, on the same bf16 values) for the query heads with the fewest and
+    the most kept blocks: mismatches, and how many of them the contract allows (within 1e-5 of tau, or runs of
+    equal sums cut by the crossing).  The mask compared is the product path's (normalise-and-select pass)."""
+    from oracle.parity import head_mask_parity
+    from xattn.src.Xattention import estimate_and_select
+
+    kept = col_cnt.long().sum(-1)
+    heads = sorted({int(kept.argmin()), int(kept.argmax())})
+    r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, want_lists=False, want_sums=False)
+    tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "ties": 0, "outside_band": 0}
+    for h in heads:
+        rep = head_mask_parity(q, k, h, r["mask"][h], w.stride, tau, chunk, w.causal, pad0_quirk=False)
+        for key in tot:
+            tot[key] += rep[key]
+    tot["heads"] = heads
+    return tot
+
+
+def summarize(w, L, tau, chunk, m, headline_traffic=False):
+    """The per-workload numbers of the JSON line from measure()'s samples."""
+    fb = flops_and_bytes(w, L, chunk, m["n_sel"])
+    t_est, t_sel, t_att = statistics.mean(m["est"]), statistics.mean(m["sel"]), statistics.mean(m["att"])
+    t_tot, t_dense = statistics.mean(m["tot"]), statistics.median(m["dense"])
+    est_tf = fb["f_est"] / (t_est * 1e-3) / 1e12
+    att_tf = fb["f_sparse"] / (t_att * 1e-3) / 1e12
+    rl_est = {
+        "kernel": "estimate_gemm_kernel", "bound": "mfma", "achieved": round(est_tf, 1), "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(est_tf / PEAK_BF16_TFLOPS, 4), "ms": round(t_est, 3), "flop": fb["f_est"],
+        "traffic": measured_traffic_bytes("xattn::estimate_gemm_kernel") if headline_traffic else None,
+    }
+    rl_att = {
+        "kernel": "block_sparse_fwd_kernel<true>", "bound": "mfma", "achieved": round(att_tf, 1),
+        "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(att_tf / PEAK_BF16_TFLOPS, 4), "ms": round(t_att, 3),
+        "flop": fb["f_sparse"],
+        "traffic": measured_traffic_bytes("xattn::block_sparse_fwd_kernel<true>") if headline_traffic else None,
+    }
+    sel_gbs = fb["pass_bytes"] / (t_sel * 1e-3) / 1e9
+    rl_sel = {
+        "kernel": "estimate_select_kernel (normalisation + selection, block sums in LDS)", "bound": "hbm",
+        "achieved": round(sel_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(sel_gbs / PEAK_HBM_GBS, 4),
+        "ms": round(t_sel, 3), "bytes": fb["pass_bytes"],
+        "reference_staging_bytes": fb["survey_bytes"],     # full block-sum matrix in, byte mask + lists out
+        "traffic": measured_traffic_bytes("xattn::estimate_select_kernel") if headline_traffic else None,
+    }
+    return {
+        "estimate_ms": round(t_est, 3), "select_ms": round(t_sel, 3), "sparse_attn_ms": round(t_att, 3),
+        "total_ms": round(t_tot, 3), "total_ms_stats": _stats(m["tot"]),
+        "estimate_ms_stats": _stats(m["est"]), "select_ms_stats": _stats(m["sel"]), "sparse_attn_ms_stats": _stats(m["att"]),
+        "dense_fa_ms": round(t_dense, 3), "dense_fa_ms_stats": _stats(m["dense"]),
+        "speedup_vs_dense_fa": round(t_dense / t_tot, 3),
+        "estimate_fraction_of_total": round((t_est + t_sel) / t_tot, 4),
+        "sparsity": round(1.0 - m["n_sel"] / fb["full_blocks"], 4), "selected_blocks": m["n_sel"],
+        "estimate_tflops": round(est_tf, 1), "sparse_tflops": round(att_tf, 1),
+        "dense_fa_tflops": round(fb["f_dense"] / (t_dense * 1e-3) / 1e12, 1),
+        "select_gbs": round(sel_gbs, 1),
+        "roofline_estimator": rl_est, "roofline_sparse_attention": rl_att, "roofline_select": rl_sel,
+    }
+
+
+def workload_config(w, L, tau, chunk, rank8="head"):
+    return {
+        "workload": (w.name if L == w.L else f"{w.name}@L={L}") + ("" if rank8 == "head" else "@rank8=token"),
+        "seq_len": L, "q_heads": w.heads, "kv_heads": w.kv_heads, "head_dim": 128, "stride": w.stride,
+        "threshold": tau, "chunk_size": chunk, "block_size": 128, "causal": w.causal,
+        "estimator_semantics": "all earlier keys visible (reference Triton branch)",
+    }
+
+
 def density_sweep(w, L, chunk, dev, t_dense, qkv, steps=3):
     """The headline shape at other operating points, so that estimate share and speedup are read against a range
     of densities: thresholds 0.9 / 0.95 / 0.99 on the workload's inputs, and the per-token reading of the rank-8
-    term (diffuse attention) at 0.9.  Same timing protocol as the headline, fewer steps."""
+    term (diffuse attention) at 0.9.  Same stages as the headline, fewer steps."""
     import torch
-    from xattn.src.Xattention import block_sparse_attention, estimate_and_select
     from xattn.synthetic import make_inputs
 
     rows = []
-    nb = (L + 127) // 128
-    full_blocks = w.heads * nb * (nb + 1) // 2
-    n_r = ((L + chunk - 1) // chunk * chunk) // w.stride
-    f_est = 2.0 * w.stride * 128 * w.heads * n_r * (n_r + 1) / 2
     for rank8, taus in (("head", (0.9, 0.95, 0.99)), ("token", (0.9,))):
         q, k, v = qkv if rank8 == "head" else make_inputs(w, device=dev, seed=0, L=L, dtype=torch.bfloat16, rank8=rank8)
         for tau in taus:
-            for i in range(steps + 1):
-                marks = []
-                r = estimate_and_select(q, k, w.stride, tau, chunk, causal=True, marks=marks, want_mask=False)
-                block_sparse_attention(q, k, v, r["col_idx"], r["col_cnt"], causal=True)
-                end = torch.cuda.Event(enable_timing=True)
-                end.record()
-                torch.cuda.synchronize()
-                m = dict(marks)
-                if i == 0:
-                    acc = [0.0, 0.0, 0.0]
-                    continue
-                acc[0] += _ms(m["estimate_begin"], m["select_begin"]) / steps
-                acc[1] += _ms(m["select_begin"], m["select_end"]) / steps
-                acc[2] += _ms(m["select_end"], end) / steps
-            n_sel = int(r["col_cnt"][:, :nb].sum().item())
-            total = sum(acc)
+            m = measure(w, q, k, v, L, tau, chunk, steps, 1, 0, 0)
+            fb = flops_and_bytes(w, L, chunk, m["n_sel"])
+            t_est, t_sel, t_att = statistics.mean(m["est"]), statistics.mean(m["sel"]), statistics.mean(m["att"])
+            total = t_est + t_sel + t_att
             rows.append({
-                "rank8": rank8, "threshold": tau, "density": round(n_sel / full_blocks, 4),
-                "estimate_ms": round(acc[0], 3), "select_ms": round(acc[1], 3), "sparse_attn_ms": round(acc[2], 3),
-                "total_ms": round(total, 3), "estimate_share": round((acc[0] + acc[1]) / total, 4),
-                "estimate_pflops": round(f_est / (acc[0] * 1e-3) / 1e15, 3),
-                "sparse_pflops": round(4.0 * 128 ** 3 * n_sel / (acc[2] * 1e-3) / 1e15, 3),
+                "rank8": rank8, "threshold": tau, "density": round(m["n_sel"] / fb["full_blocks"], 4),
+                "estimate_ms": round(t_est, 3), "select_ms": round(t_sel, 3), "sparse_attn_ms": round(t_att, 3),
+                "total_ms": round(total, 3), "estimate_share": round((t_est + t_sel) / total, 4),
+                "estimate_pflops": round(fb["f_est"] / (t_est * 1e-3) / 1e15, 3),
+                "sparse_pflops": round(fb["f_sparse"] / (t_att * 1e-3) / 1e15, 3),
                 "speedup_vs_dense_fa": round(t_dense / total, 2),
             })
         del q, k, v
     return rows
 
 
+def yardsticks(dev):
+    """Two library kernels of known provenance on the same box, measurement only (nothing in the package uses
+    them): torch.matmul (hipBLASLt) on a bf16 GEMM of the estimator's per-head shape - reshaped length 8192,
+    depth stride * 128 = 2048, the full square, i.e. twice the causal estimator's flops per head - called 32
+    times back to back like the 32 heads; and torch's flash scaled_dot_product_attention, causal, 32 heads,
+    L = 32768 (workload 1's shape with K/V repeated to 32 heads).  The batched form of the GEMM
+    ([32, 8192, 2048] x [32, 2048, 8192], a 4 GiB result) is not used: that call ended in an illegal memory
+    access inside the library on this image."""
+    import torch
+    import torch.nn.functional as F
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    def timed(fn, warm, reps):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(_ms(e0, e1))
+        return ts
+
+    res = {}
+    with torch.no_grad():
+        a = torch.randn(8192, 2048, device=dev).bfloat16()
+        b = torch.randn(8192, 2048, device=dev).bfloat16()
+
+        def gemm32():
+            for _ in range(32):
+                torch.matmul(a, b.t())
+
+        ts = timed(gemm32, 2, 5)
+        fl = 32 * 2.0 * 8192 * 8192 * 2048
+        res["gemm_bf16_8192x8192x2048_x32"] = {
+            "library": "torch.matmul (hipBLASLt)", "ms": _stats(ts), "tflops": round(fl / (statistics.median(ts) * 1e-3) / 1e12, 1)}
+        del a, b
+        L = 32768
+        try:
+            q = torch.randn(1, 32, L, 128, device=dev).bfloat16()
+            k = torch.randn(1, 32, L, 128, device=dev).bfloat16()
+            v = torch.randn(1, 32, L, 128, device=dev).bfloat16()
+            with sdpa_kernel(SDPBackend.FLASH_ATTENTION):
+                ts = timed(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True), 1, 3)
+            fl = 4.0 * 128 * 32 * L * (L + 1) / 2
+            res["sdpa_flash_causal_L32768_h32"] = {
+                "library": "torch scaled_dot_product_attention, FLASH_ATTENTION backend", "ms": _stats(ts),
+                "tflops": round(fl / (statistics.median(ts) * 1e-3) / 1e12, 1)}
+            del q, k, v
+        except Exception as e:      # the backend may refuse the call on another build; the GEMM figure stands alone then
+            res["sdpa_flash_causal_L32768_h32"] = {"error": f"{type(e).__name__}: {str(e)[:200]}"}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", type=int, default=2, help="index into the synthetic workloads (default: headline)")
-    ap.add_argument("--dense-steps", type=int, default=2)
+    ap.add_argument("--dense-steps", type=int, default=5)
+    ap.add_argument("--dense-warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode-step measurement")
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only rate probe")
+    ap.add_argument("--no-workloads", action="store_true", help="skip the measurements of the other GPU workloads")
+    ap.add_argument("--no-yardsticks", action="store_true", help="skip the library GEMM / flash attention yardsticks")
     ap.add_argument("--compare-pipelined", action="store_true",
                     help="also time Xattention_prefill with and without chunk-by-chunk stream pipelining")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -246,7 +463,7 @@ def main():
                     help="reading of the text workloads' shared rank-8 component (see xattn/synthetic.py)")
     ap.add_argument("--no-density-sweep", action="store_true",
                     help="skip the extra timings of the headline shape at other thresholds / the per-token generator")
-    ap.add_argument("--no-mask-parity", action="store_true", help="skip the oracle run on two heads of the workload")
+    ap.add_argument("--no-mask-parity", action="store_true", help="skip the oracle runs on two heads of each workload")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the prefill path uses no collectives; run with --gpus 1", file=sys.stderr)
@@ -270,132 +487,43 @@ def main():
     chunk = w.chunk_size or default_chunk_size(L)
     torch.cuda.synchronize()
 
-    def step(marks=None):
-        # what the operator itself runs: column lists only, no byte mask
-        r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, marks=marks, want_mask=False)
-        if marks is not None:
-            marks.append(("sparse_begin", marks[-1][1]))
-        out = block_sparse_attention(q, k, v, r["col_idx"], r["col_cnt"], causal=w.causal)
-        if marks is not None:
-            ev = torch.cuda.Event(enable_timing=True)
-            ev.record()
-            marks.append(("sparse_end", ev))
-        return r, out
-
-    with torch.no_grad():
-        for _ in range(args.warmup):
-            r, out = step()
-        torch.cuda.synchronize()
-        all_marks = []
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            m = []
-            r, out = step(m)
-            all_marks.append(dict(m))
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-
-        t_est = statistics.mean(_ms(m["estimate_begin"], m["select_begin"]) for m in all_marks)
-        t_sel = statistics.mean(_ms(m["select_begin"], m["select_end"]) for m in all_marks)
-        t_sparse = statistics.mean(_ms(m["sparse_begin"], m["sparse_end"]) for m in all_marks)
-        t_total = statistics.mean(_ms(m["estimate_begin"], m["sparse_end"]) for m in all_marks)
-
-        # dense causal FlashAttention written the same way (same kernel, every visible block)
-        block_sparse_attention(q, k, v, causal=w.causal)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(args.dense_steps):
-            dense = block_sparse_attention(q, k, v, causal=w.causal)
-        e1.record()
-        torch.cuda.synchronize()
-        t_dense = _ms(e0, e1) / args.dense_steps
-
-    nb = (L + 127) // 128
-    n_sel = int(r["col_cnt"][:, :nb].sum().item())
-    H = w.heads
-    full_blocks = H * nb * (nb + 1) // 2 if w.causal else H * nb * nb
-    sparsity = 1.0 - n_sel / full_blocks
-    f_sparse = 4.0 * 128 * 128 * 128 * n_sel
-    f_dense = (4.0 * 128 * H * L * (L + 1) / 2) if w.causal else (4.0 * 128 * H * L * L)
-    n_r = ((L + chunk - 1) // chunk * chunk) // w.stride
-    f_est = (2.0 * w.stride * 128 * H * n_r * (n_r + 1) / 2) if w.causal else (2.0 * w.stride * 128 * H * n_r * n_r)
-    nkb_p = (L + chunk - 1) // chunk * chunk // 128
-    sel_bytes = H * nkb_p * nkb_p * 5 + 4 * (n_sel + H * nkb_p)
-    sparse_tflops = f_sparse / (t_sparse * 1e-3) / 1e12
-    est_tflops = f_est / (t_est * 1e-3) / 1e12
+    m = measure(w, q, k, v, L, tau, chunk, args.steps, args.warmup, args.dense_steps, args.dense_warmup)
     as_configured = L == w.L and args.threshold is None and args.rank8 == "head"
-    headline_traffic = as_configured and w.name == HEADLINE
-    roofline_sparse = {
-        "kernel": "block_sparse_fwd_kernel<true>", "bound": "mfma", "achieved": round(sparse_tflops, 1),
-        "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(sparse_tflops / PEAK_BF16_TFLOPS, 4),
-        "ms": round(t_sparse, 3), "flop": f_sparse,
-        "traffic": measured_traffic_bytes("xattn::block_sparse_fwd_kernel<true>") if headline_traffic else None,
-    }
-    # the estimator stage is one entry point = the MFMA kernel plus its short normalisation pass (about 6 % of the
-    # stage at the headline); its time is taken between the same stream events
-    roofline_est = {
-        "kernel": "estimate_gemm_kernel (+ estimate_normalize_kernel, same entry point)", "bound": "mfma",
-        "achieved": round(est_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(est_tflops / PEAK_BF16_TFLOPS, 4), "ms": round(t_est, 3), "flop": f_est,
-        "traffic": measured_traffic_bytes("xattn::estimate_gemm_kernel") if headline_traffic else None,
-    }
-    dominant = roofline_est if t_est >= t_sparse else roofline_sparse
+    is_headline = as_configured and w.name == HEADLINE
+    head = summarize(w, L, tau, chunk, m, headline_traffic=is_headline)
+    rl_est, rl_att = head["roofline_estimator"], head["roofline_sparse_attention"]
+    dominant = rl_est if rl_est["ms"] >= rl_att["ms"] else rl_att
 
     result = {
         "metric": "per-layer prefill attn ms (estimate+sparse) at 128k; speedup vs dense FA",
-        "value": round(t_total, 3),
+        "value": head["total_ms"],
         "unit": "ms",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 3),
+        "ms_per_step": round(m["wall_ms"], 3),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {
-            "workload": (w.name if L == w.L else f"{w.name}@L={L}") + ("" if args.rank8 == "head" else "@rank8=token"),
-            "seq_len": L, "q_heads": H, "kv_heads": w.kv_heads, "head_dim": 128, "stride": w.stride,
-            "threshold": tau, "chunk_size": chunk, "block_size": 128, "causal": w.causal,
-            "estimator_semantics": "all earlier keys visible (reference Triton branch)",
-        },
-        "estimate_ms": round(t_est, 3),
-        "select_ms": round(t_sel, 3),
-        "sparse_attn_ms": round(t_sparse, 3),
-        "dense_fa_ms": round(t_dense, 3),
-        "speedup_vs_dense_fa": round(t_dense / t_total, 3),
-        "estimate_fraction_of_total": round((t_est + t_sel) / t_total, 4),
-        "sparsity": round(sparsity, 4),
-        "selected_blocks": n_sel,
-        "estimate_tflops": round(est_tflops, 1),
-        "dense_fa_tflops": round(f_dense / (t_dense * 1e-3) / 1e12, 1),
-        "select_gbs": round(sel_bytes / (t_sel * 1e-3) / 1e9, 1),
-        # the launch that takes longest of the two MFMA stages; both are listed after it
-        "roofline": dict(dominant),
-        "roofline_estimator": roofline_est,
-        "roofline_sparse_attention": roofline_sparse,
+        "config": workload_config(w, L, tau, chunk, args.rank8),
+        "timing": {"warmup_steps": args.warmup, "timed_steps": args.steps, "value_is": "mean of the timed steps",
+                   "dense_warmup": args.dense_warmup, "dense_timed": args.dense_steps, "dense_fa_ms_is": "median",
+                   "stages": "estimate_ms = the estimator's MFMA pass (estimate_gemm_kernel), select_ms = its normalisation "
+                             "fused with the block selection (estimate_select_kernel), sparse_attn_ms = block_sparse_fwd_kernel"},
+        "kernel_sources_sha256_16": kernel_source_hash(),
     }
-    del dense, out
-    if not args.no_mask_parity and w.causal is not None:
-        # block-mask parity with the oracle (fp32, on the same bf16 values) for the query heads with the fewest and
-        # the most kept blocks: mismatches, and how many of them the contract allows (within 1e-5 of tau, or runs of
-        # equal sums cut by the crossing)
-        from oracle.parity import head_mask_parity
-
-        kept = r["col_cnt"].long().sum(-1)
-        heads = sorted({int(kept.argmin()), int(kept.argmax())})
-        r = estimate_and_select(q, k, w.stride, tau, chunk, causal=w.causal, want_lists=False)     # with the mask
-        tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "ties": 0, "outside_band": 0}
-        for h in heads:
-            rep = head_mask_parity(q, k, h, r["mask"][h], w.stride, tau, chunk, w.causal, pad0_quirk=False)
-            for key in tot:
-                tot[key] += rep[key]
-        tot["heads"] = heads
-        result["mask_parity"] = tot
-    if (not args.no_density_sweep) and as_configured and w.name == HEADLINE:
-        result["density_sweep"] = density_sweep(w, L, chunk, dev, t_dense, (q, k, v))
+    result.update({key: val for key, val in head.items() if not key.startswith("roofline_")})
+    # the launch that takes longest of the two MFMA stages; both are listed after it, and the selection pass
+    result["roofline"] = dict(dominant)
+    result["roofline_estimator"] = rl_est
+    result["roofline_sparse_attention"] = rl_att
+    result["roofline_select"] = head["roofline_select"]
+    if not args.no_mask_parity:
+        result["mask_parity"] = mask_parity(w, q, k, tau, chunk, m["col_cnt"])
+    if (not args.no_density_sweep) and is_headline:
+        result["density_sweep"] = density_sweep(w, L, chunk, dev, head["dense_fa_ms"], (q, k, v))
     if args.compare_pipelined:
         from xattn.src.Xattention import Xattention_prefill
 
@@ -425,6 +553,30 @@ def main():
         del src, dst
     if not args.no_decode:
         result["decode_step"] = decode_leg(q, k, v)
+    del q, k, v, m
+    torch.cuda.empty_cache()
+    if (not args.no_workloads) and is_headline:
+        # the other GPU workloads, same protocol with fewer steps (their launches are up to 20x longer)
+        others = []
+        for idx in (1, 3, 4):
+            w2 = WORKLOADS[idx]
+            c2 = w2.chunk_size or default_chunk_size(w2.L)
+            q2, k2, v2 = make_inputs(w2, device=dev, seed=0, L=w2.L, dtype=torch.bfloat16)
+            steps2 = 30 if idx == 1 else 10
+            m2 = measure(w2, q2, k2, v2, w2.L, w2.threshold, c2, steps2, 10 if idx == 1 else 3, 5 if idx == 1 else 3, 1)
+            row = {"config": workload_config(w2, w2.L, w2.threshold, c2), "steps": steps2}
+            s2 = summarize(w2, w2.L, w2.threshold, c2, m2)
+            for key in ("roofline_estimator", "roofline_sparse_attention", "roofline_select"):
+                s2[key] = {kk: vv for kk, vv in s2[key].items() if kk in ("kernel", "achieved", "unit", "frac", "ms")}
+            row.update(s2)
+            if not args.no_mask_parity:
+                row["mask_parity"] = mask_parity(w2, q2, k2, w2.threshold, c2, m2["col_cnt"])
+            others.append(row)
+            del q2, k2, v2, m2
+            torch.cuda.empty_cache()
+        result["workloads"] = others
+    if not args.no_yardsticks:
+        result["yardsticks"] = yardsticks(dev)
     if not args.no_mfma_probe:
         result["mfma_alone"] = mfma_probe(dev)
     if not args.no_cpu_baseline:
