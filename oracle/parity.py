@@ -108,7 +108,8 @@ def mask_mismatch_report(sums, got, want, tau, causal, diag_offset, blocks_per_c
     return d["mismatches"], d["outside"]
 
 
-def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal, pad0_quirk, sums_got=None):
+def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal, pad0_quirk, sums_got=None,
+                     return_mask=False):
     """Runs the oracle's estimate for ONE query head on the host, in fp32, on the
     values ``q``/``k`` hold (any dtype/device; K may carry fewer heads), and
     compares its block mask with ``got_mask`` (that head's ``[Nq_p, Nk_p]`` mask
@@ -117,7 +118,8 @@ def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal
     Returns a dict: blocks, mismatches, in_band and ties (mismatches the contract
     allows), outside_band, density of the oracle's mask over the padded grid
     and, when ``sums_got`` is given, the largest absolute difference of the
-    block sums.
+    block sums; with ``return_mask`` also the oracle's mask for the head
+    (``oracle_mask``, bool ``[Nq_p, Nk_p]``).
     """
     H, Hkv = q.shape[1], k.shape[1]
     kv = head // (H // Hkv)
@@ -136,4 +138,6 @@ def head_mask_parity(q, k, head, got_mask, stride, threshold, chunk_size, causal
            "ties": d["ties"], "outside_band": d["outside"], "oracle_density": round(float(want_mask.float().mean()), 5)}
     if sums_got is not None:
         rep["sums_max_abs_diff"] = float((sums_got.detach().float().cpu().reshape(nq_p, nk_p) - want_sums[0, 0]).abs().max())
+    if return_mask:
+        rep["oracle_mask"] = want_mask[0, 0].clone()
     return rep

@@ -100,3 +100,14 @@ def test_rejects_bad_arguments():
         block_sparse_attention(q.cuda().float(), k.cuda(), v.cuda())
     with pytest.raises(hb.XattnHipError):
         block_sparse_attention(q, k, v)  # CPU tensors: no fallback
+    # lists that cover only some q-blocks and no buffer to fill: refused (a fresh output would keep
+    # uninitialised rows); with the buffer and the range it is the chunk-by-chunk form
+    q, k, v = _mk(2, 2, 512, 512, 1)
+    idx = torch.zeros(2, 2, 4, dtype=torch.int32, device="cuda")
+    cnt = torch.ones(2, 2, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        block_sparse_attention(q.cuda(), k.cuda(), v.cuda(), idx, cnt)
+    out = torch.zeros(1, 512, 2, 128, dtype=torch.bfloat16, device="cuda")
+    block_sparse_attention(q.cuda(), k.cuda(), v.cuda(), idx, cnt, out=out, q_blocks=(0, 2))
+    torch.cuda.synchronize()
+    assert out[0, :256].float().abs().sum() > 0 and out[0, 256:].float().abs().sum() == 0

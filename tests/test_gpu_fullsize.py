@@ -76,10 +76,16 @@ def test_full_size_workload_properties(idx):
 
     out = block_sparse_attention(q, k, v, idx_t, cnt, causal=w.causal)
     assert torch.isfinite(out.float()).all()
+    # deterministic samples: the (head, q-block) with the longest list, the median one, the first and the last
+    # (ragged for workload 4) q-block, and one q-block of every KV group
+    lens = cnt[:, :nb].long().reshape(-1).cpu()
+    order = torch.argsort(lens)
+    samples = [divmod(int(order[-1]), nb), divmod(int(order[len(order) // 2]), nb), (0, 0), (H - 1, nb - 1)]
+    group = H // w.kv_heads
     g = torch.Generator().manual_seed(idx)
-    samples = [(int(torch.randint(H, (1,), generator=g)), int(torch.randint(nb, (1,), generator=g))) for _ in range(3)]
-    samples += [(0, 0), (H - 1, nb - 1)]
-    _sampled_block_parity(q, k, v, mask, out, w.causal, samples)
+    for kvh in range(w.kv_heads):
+        samples.append((kvh * group + int(torch.randint(group, (1,), generator=g)), int(torch.randint(nb, (1,), generator=g))))
+    _sampled_block_parity(q, k, v, mask, out, w.causal, sorted(set(samples)))
     density = cnt[:, :nb].sum().item() / (H * (nb * (nb + 1) // 2 if w.causal else nb * nb))
     print(f"{w.name}: density {density:.4f}")
 

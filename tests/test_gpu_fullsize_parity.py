@@ -11,7 +11,8 @@ configuration) is run on its bf16 cast for all 32 heads.
 import pytest
 import torch
 
-from helpers import head_mask_parity
+from helpers import OUT_MAX_ABS, OUT_MEAN_ABS, head_mask_parity, lists_from_mask
+from oracle import xattn_oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -19,11 +20,42 @@ SUMS_ATOL = 2e-5
 SUMS_RTOL = 2e-4
 
 
-def _check_heads(w, q, k, r, heads, chunk, use_triton):
+def _attention_under_oracle_mask(w, q, k, v, h, oracle_mask):
+    """Attention output of head h computed by the kernel FROM THE ORACLE'S MASK (as column lists), against the
+    oracle's masked dense attention on the q-blocks with the longest list, the median one and the last
+    (possibly ragged) one.  Tolerance of the parity contract: 2e-2 max-abs, 5e-3 mean-abs."""
+    from xattn.src.Xattention import block_sparse_attention
+
+    L = q.shape[2]
+    nb = (L + 127) // 128
+    kv = h // (w.heads // w.kv_heads)
+    m = oracle_mask[:nb, :nb]
+    idx, cnt = lists_from_mask(m[None])
+    out = block_sparse_attention(q[:, h : h + 1], k[:, kv : kv + 1], v[:, kv : kv + 1], idx.cuda(), cnt.cuda(), causal=w.causal)
+    torch.cuda.synchronize()
+    lens = cnt[0].long()
+    order = torch.argsort(lens)
+    picks = sorted({int(order[-1]), int(order[len(order) // 2]), nb - 1})
+    for qb in picks:
+        r0, r1 = qb * 128, min(L, qb * 128 + 128)
+        kend = r1 if w.causal else L
+        nkb = (kend + 127) // 128
+        want = O.block_sparse_attention(q[:, h : h + 1, r0:r1].float().cpu(), k[:, kv : kv + 1, :kend].float().cpu(),
+                                        v[:, kv : kv + 1, :kend].float().cpu(), m[qb : qb + 1, :nkb][None, None], causal=w.causal)
+        err = (out[:, :, r0:r1].float().cpu() - want).abs()
+        print(f"{w.name} head {h} q-block {qb} ({int(lens[qb])} blocks): max {err.max().item():.4f} mean {err.mean().item():.5f}",
+              flush=True)
+        assert err.max().item() <= OUT_MAX_ABS, (h, qb, err.max().item())
+        assert err.mean().item() <= OUT_MEAN_ABS, (h, qb, err.mean().item())
+
+
+def _check_heads(w, q, k, r, heads, chunk, use_triton, v=None):
     tot = {"blocks": 0, "mismatches": 0, "in_band": 0, "ties": 0, "outside_band": 0}
     for h in heads:
         rep = head_mask_parity(q, k, h, r["mask"][h], w.stride, w.threshold, chunk, w.causal,
-                               pad0_quirk=not use_triton, sums_got=r["sums"][h])
+                               pad0_quirk=not use_triton, sums_got=r["sums"][h], return_mask=v is not None)
+        if v is not None:
+            _attention_under_oracle_mask(w, q, k, v, h, rep.pop("oracle_mask"))
         print(f"{w.name} use_triton={use_triton} {rep}", flush=True)
         for key in tot:
             tot[key] += rep[key]
@@ -39,7 +71,7 @@ def test_mask_parity_at_benchmark_size(idx, use_triton):
     from xattn.synthetic import WORKLOADS, make_inputs
 
     w = WORKLOADS[idx]
-    q, k, _ = make_inputs(w, device="cuda", seed=0)
+    q, k, v = make_inputs(w, device="cuda", seed=0)
     chunk = w.chunk_size or default_chunk_size(w.L)
     r = estimate_and_select(q, k, w.stride, w.threshold, chunk, causal=w.causal, use_triton=use_triton)
     torch.cuda.synchronize()
@@ -47,7 +79,8 @@ def test_mask_parity_at_benchmark_size(idx, use_triton):
     heads = sorted({int(kept.argmin()), int(kept.argmax())})
     if len(heads) == 1:
         heads.append((heads[0] + 1) % w.heads)
-    tot = _check_heads(w, q, k, r, heads, chunk, use_triton)
+    # with the production semantics, also the attention output under the ORACLE's mask for those heads
+    tot = _check_heads(w, q, k, r, heads, chunk, use_triton, v=v if use_triton else None)
     print(f"{w.name} use_triton={use_triton}: heads {heads} total {tot}", flush=True)
 
 

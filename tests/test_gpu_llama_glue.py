@@ -51,14 +51,15 @@ def test_full_metric_prefill_and_decode_match_stock_attention():
             nxt = a.logits[:, -1:].argmax(-1)
 
 
-def test_static_cache_is_cut_to_its_filled_part():
+@pytest.mark.parametrize("mode", [torch.no_grad, torch.inference_mode])
+def test_static_cache_is_cut_to_its_filled_part(mode):
     from transformers import StaticCache
     from xattn.src.load_llama import FastPrefillConfig, patch_model
 
     stock = _tiny_llama(5)
     ours = patch_model(copy.deepcopy(stock), FastPrefillConfig(threshold=0.9, metric="full"))
     ids = torch.randint(0, 512, (1, 700), generator=torch.Generator().manual_seed(6)).cuda()
-    with torch.no_grad():
+    with mode():
         a = stock(ids, use_cache=True)                              # growing cache
         cache = StaticCache(config=ours.config, max_cache_len=1024)
         b = ours(ids, past_key_values=cache, use_cache=True)        # preallocated cache, 1024 slots

@@ -89,3 +89,57 @@ def test_rotary_matches_model_code():
     a = apply_rotary_pos_emb(q, k, ang.cos(), ang.sin())
     b = m.apply_rotary_pos_emb(q, k, ang.cos(), ang.sin())
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+@pytest.mark.parametrize("mode", [torch.no_grad, torch.inference_mode])
+def test_static_cache_branch_on_the_host(monkeypatch, mode):
+    """The preallocated-cache branch of the forward (how much of the cache is filled) with the attention kernels
+    replaced by torch reference attention, so that it runs without a GPU: under ``torch.inference_mode()``
+    tensors carry no version counter, and the positions may come as ``cache_position`` or ``position_ids``."""
+    import copy
+
+    import torch.nn.functional as F
+    from transformers import LlamaConfig, StaticCache
+    from transformers.models.llama.modeling_llama import LlamaForCausalLM
+
+    from xattn.src import load_llama
+    from xattn.src.load_llama import FastPrefillConfig, patch_model
+
+    def attention(q, k, v, causal=True, **kw):
+        rep = q.shape[1] // k.shape[1]
+        k, v = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
+        lq, lk = q.shape[2], k.shape[2]
+        mask = torch.ones(lq, lk, dtype=torch.bool).tril(lk - lq)
+        return F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+
+    def decode(q, k, v, kv_layout="HND", **kw):
+        return attention(q[None, :, None, :], k[None], v[None])[0, :, 0]
+
+    monkeypatch.setattr(load_llama, "block_sparse_attention", attention)
+    monkeypatch.setattr(load_llama, "single_decode_with_kv_cache", decode)
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=128, hidden_size=256, intermediate_size=256, num_hidden_layers=2, num_attention_heads=2,
+                      num_key_value_heads=1, head_dim=128, max_position_embeddings=512, attn_implementation="eager")
+    stock = LlamaForCausalLM(cfg).eval()
+    ours = patch_model(copy.deepcopy(stock), FastPrefillConfig(threshold=0.9, metric="full"))
+    ids = torch.randint(0, 128, (1, 40), generator=torch.Generator().manual_seed(1))
+    with mode():
+        a = stock(ids, use_cache=True)
+        cache = StaticCache(config=ours.config, max_cache_len=64)
+        b = ours(ids, past_key_values=cache, use_cache=True)
+        assert torch.allclose(b.logits, a.logits, atol=1e-4, rtol=1e-4)
+        nxt = a.logits[:, -1:].argmax(-1)
+        for step in range(2):
+            a = stock(nxt, past_key_values=a.past_key_values, use_cache=True)
+            b = ours(nxt, past_key_values=cache, use_cache=True)
+            assert torch.allclose(b.logits, a.logits, atol=1e-4, rtol=1e-4), step
+            nxt = a.logits[:, -1:].argmax(-1)
+    # positions through position_ids only (an attention layer called without cache_position)
+    layer = ours.model.layers[0].self_attn
+    with mode():
+        cache2 = StaticCache(config=ours.config, max_cache_len=64)
+        h = torch.randn(1, 10, 256)
+        pos = torch.arange(10)[None]
+        cos, sin = ours.model.rotary_emb(h, pos)
+        out = layer(h, position_embeddings=(cos, sin), past_key_values=cache2, position_ids=pos)[0]
+        assert out.shape == (1, 10, 256) and torch.isfinite(out).all()

@@ -66,3 +66,31 @@ def test_static_decode_through_the_python_wrapper_and_its_limit():
     assert big == -7 and b"workspace" in lib.xattn_error_string(big)
     assert lib.xattn_decode_fwd_static(None, k.data_ptr(), v.data_ptr(), out.data_ptr(), 16, 4, 5000, 128,
                                        128, 128, 512, 128, 512, 128, 0.1, None) == -1
+
+
+def test_static_decode_replays_from_a_graph():
+    """What the entry point is for: a capture refuses allocations (hipMalloc inside a capturing stream is an
+    error), so a graph that holds the static form and replays correctly shows that it allocates nothing -
+    which the allocator statistics above cannot (they only see torch's own allocator)."""
+    from xattn.src.decode import single_decode_with_kv_cache
+
+    H, Hkv, L = 32, 8, 6000
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randn(H, 128, device="cuda", generator=g).bfloat16()
+    k = torch.randn(Hkv, L, 128, device="cuda", generator=g).bfloat16()
+    v = torch.randn(Hkv, L, 128, device="cuda", generator=g).bfloat16()
+    out = torch.empty(H, 128, dtype=torch.bfloat16, device="cuda")
+    single_decode_with_kv_cache(q, k, v, "HND", out=out, static_scratch=True)   # the symbol lookup happens here
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        single_decode_with_kv_cache(q, k, v, "HND", out=out, static_scratch=True)
+    for i in range(3):
+        q.copy_(torch.randn(H, 128, device="cuda", generator=g).bfloat16())
+        v[:, i * 50:(i + 1) * 50].mul_(2.0)                                      # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = single_decode_with_kv_cache(q, k, v, "HND")                       # the workspace form, eager
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), i

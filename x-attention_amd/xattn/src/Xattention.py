@@ -413,6 +413,7 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
         raise AssertionError("key_states and value_states must agree in heads and length")
     if (col_idx is None) != (col_cnt is None):
         raise AssertionError("col_idx and col_cnt go together")
+    out_given = out is not None
     if out is None:
         out = torch.empty((1, q_len, heads, 128), dtype=torch.bfloat16, device=dev)
     qb0, qb1 = q_blocks if q_blocks is not None else (0, -1)
@@ -424,6 +425,11 @@ def block_sparse_attention(query_states, key_states, value_states, col_idx=None,
         pitch, idx_rows = col_idx.shape[2], col_idx.shape[1]
         if q_blocks is None:
             qb0, qb1 = idx_row0, min((q_len + 127) // 128, idx_row0 + idx_rows)
+            if out_given is False and (qb0 != 0 or qb1 != (q_len + 127) // 128):
+                # lists that cover only some q-blocks fill only those rows of the output: a caller who means
+                # that passes the buffer to fill (and usually q_blocks); a fresh buffer would come back with
+                # uninitialised rows
+                raise ValueError("col_idx / col_cnt do not cover every q-block: pass `out` (and `q_blocks`) to fill part of it")
     else:
         pitch, idx_rows = 0, 0
     with torch.cuda.device(dev):

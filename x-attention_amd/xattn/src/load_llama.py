@@ -142,14 +142,15 @@ def forward_eval(self, hidden_states, position_embeddings=None, attention_mask=N
             pos = cache_position if cache_position is not None else (position_ids[0] if position_ids is not None else None)
             if pos is None:
                 raise ValueError("a static cache needs cache_position or position_ids to know how much of it is filled")
-            # reading the position costs a device-to-host copy: do it once per model forward (every layer is
-            # handed the same tensor object), not once per layer
+            # reading the position costs a device-to-host copy: the first layer of a model forward does it, the
+            # other layers (handed the same positions) reuse its value.  Nothing here depends on tensor
+            # identity or version counters, which inference-mode tensors do not have.
             memo = getattr(cfg, "_filled_memo", None)
-            if memo is not None and memo[0] is pos and memo[1] == pos._version:
-                last = memo[2]
-            else:
+            if memo is None or self.layer_idx in (0, None):
                 last = int(pos[-1])
-                cfg._filled_memo = (pos, pos._version, last)
+                cfg._filled_memo = (last,)
+            else:
+                last = memo[0]
             filled = min(last + 1, key_states.shape[2])
             key_states, value_states = key_states[:, :, :filled], value_states[:, :, :filled]
     if key_states.device != query_states.device:
