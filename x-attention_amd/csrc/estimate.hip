@@ -15,8 +15,9 @@
 //    block_size/S keys.  It writes, per (query row, 128-key tile), the local
 //    maximum and sum, and per (query row, key block) the partial sum - 1/S of
 //    the score matrix, in fp32 - never the scores themselves.  One workgroup
-//    per CU works through its share of the tiles with the copy pipeline
-//    running on across tile boundaries.
+//    per CU works through its share of the tiles with the slab pipeline
+//    (global -> registers -> LDS, two k-steps deep) running on across tile
+//    boundaries.
 //  kernel 2 (estimate_normalize_kernel): per query row, combines the tile
 //    maxima/sums into the row's softmax statistics, rescales the partial sums
 //    and adds the block_size/S rows of each query block.
@@ -76,18 +77,22 @@ __host__ __device__ inline int row_hi(const EstParams& p, int m) {
   return p.causal ? m * p.kdb + p.kdb - 1 + p.off : p.n_rk - 1;
 }
 
-// A k-step slab is 256 rows x 64 bf16 (one 128-byte line per row) per operand,
-// copied global -> LDS by buffer loads that write LDS directly (no register
-// staging): each wavefront instruction moves 64 x 16 bytes into one contiguous
-// KiB, i.e. 8 rows.  Tokens past the real length fall outside the buffer
-// resource and arrive as zeros - the zero padding of xattn/src/Xattention.py:33-51.
+// A k-step slab is 256 rows x 64 bf16 (one 128-byte line per row) per operand.
+// It travels global -> registers -> LDS: each wavefront instruction loads
+// 64 x 16 bytes = 8 rows (full lines) and later writes them as one contiguous
+// KiB.  Loads are issued two k-steps ahead of their use and written to LDS one
+// step ahead, so a load has a whole step to arrive and no barrier waits for
+// memory.  (Buffer loads that write LDS directly save the registers, but had
+// to be issued at most one step ahead - the stage they fill must be free -
+// and the kernel then ran 4-8 % slower.)  Tokens past the real length fall
+// outside the buffer resource and arrive as zeros - the zero padding of
+// xattn/src/Xattention.py:33-51.
 //
 // LDS slab layout: row r at byte r*128; its 16-byte chunk c sits at position
 // c ^ ((r >> 1) & 7), so the 16 lanes of one ds_read_b128 pass - the same
 // logical chunk of 16 consecutive rows - touch each of the 64 banks once.  The
 // swizzle is applied on the global side of the copy (the lane that fills
 // position c fetches chunk c ^ ((r >> 1) & 7)).
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // Per-lane byte offsets (relative to the tile's first token) of the 8 rows a
 // lane copies per slab, for token 0 of each reshaped row's group and feature 0;
@@ -99,12 +104,6 @@ __device__ __forceinline__ void slab_offsets(int64_t sn_bytes, int S, int lane, 
     const int r = it * 64 + wave * 8 + rl;
     voff[it] = (int)((int64_t)r * S * sn_bytes) + ((c ^ ((r >> 1) & 7)) << 4);
   }
-}
-
-__device__ __forceinline__ void copy_one(__amdgpu_buffer_rsrc_t rsrc, int voff, int step_off, char* slab, int wave,
-                                         int it) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(slab + (it * 64 + wave * 8) * 128), 16,
-                                           (int)((unsigned)voff + (unsigned)step_off), 0, 0, 0);
 }
 
 __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk) {
@@ -157,7 +156,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   const int r = lane & 31, hh = lane >> 5;
   const int wm = wave & 3, wn = wave >> 2;   // query quarter, key half
   // A workgroup works through tiles id, id + grid, ...: one workgroup fits a CU, so nothing else could hide
-  // the wait for a tile's first slabs.  The copy pipeline therefore runs on across the tile boundary: the copy
+  // the wait for a tile's first slabs.  The slab pipeline therefore runs on across the tile boundary: the load
   // slots of a tile's last two k-steps fetch the first slabs of the NEXT tile, and the last sub-step reads its
   // first fragments, so after the epilogue (which needs no LDS) the next tile starts at full speed.
   int64_t id = blockIdx.x;
@@ -188,14 +187,16 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   // 64*(t % 2) .. +63, and is read from LDS stage t % 2.
   //
   // Software pipeline.  A step is four sub-steps of 8 MFMAs per wavefront; the 6
-  // fragment reads of the next sub-step and 2 of the 8 copies of a later step
-  // are issued between them, in chunks the scheduler may not mix (one copy, two
-  // reads, two MFMAs), so that neither copies nor reads bunch up in front of the
-  // MFMAs.  Two wavefronts share a SIMD: while one waits at the barrier or on a
-  // fragment the other keeps the matrix pipe fed.  The workgroup barrier sits
-  // before the LAST sub-step's MFMAs: at that point every fragment of the
-  // current stage has been read, so the sub-step can prefetch the next stage's
-  // first fragments and start refilling the current stage while its MFMAs run.
+  // fragment reads of the next sub-step and up to 3 of the 8 slab pieces (an LDS
+  // write of the next step's piece, then the load of the piece two steps on
+  // into the same registers) are issued between them, in chunks the scheduler
+  // may not mix (one piece, two reads, two MFMAs), so that neither pieces nor
+  // reads bunch up in front of the MFMAs.  Two wavefronts share a SIMD: while
+  // one waits at the barrier or on a fragment the other keeps the matrix pipe
+  // fed.  The workgroup barrier sits before the LAST sub-step's MFMAs: at that
+  // point every fragment of the current stage has been read and every piece of
+  // the next stage written, so the sub-step can prefetch the next stage's first
+  // fragments while its MFMAs run.
   const int steps = (kTable ? p.n_pairs : p.S) * 2;
   int voffK[4], voffQ[4];
   slab_offsets(k_snb, p.S, lane, wave, voffK);
@@ -208,22 +209,38 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     const int i = kTable ? (p.pairs[t >> 1] >> 4) : (p.S - 1 - (t >> 1));
     return i * (int)q_snb + (t & 1) * kDepth * 2;
   };
-  // copy j (0..7) of k-step t: slab rows it = j / 2 of K' (j even) or Q' (j odd).  Steps `steps` and
-  // `steps + 1` are steps 0 and 1 of the next tile (of this tile again when it is the workgroup's last:
-  // a harmless repeat nobody reads).
-  auto copy_j = [&](int j, int t, char* stage) {
+  // Piece j (0..7) of k-step t: slab rows it = j / 2 of K' (j even) or Q' (j odd), 8 rows per wavefront.  It is
+  // loaded into R[j] during step t - 2 and written to LDS stage t % 2 during step t - 1.  Steps `steps` and
+  // `steps + 1` are steps 0 and 1 of the next tile (of this tile again when it is the workgroup's last: a harmless
+  // repeat nobody reads).
+  u32x4 R[8];
+  auto load_j = [&](int j, int t) __attribute__((always_inline)) {
     const bool ahead = t >= steps;
     const int tc = ahead ? t - steps : t;
-    if (j & 1) copy_one(ahead ? qres_next : qres, voffQ[j >> 1], step_off_q(tc), stage + kTile * 128, wave, j >> 1);
-    else copy_one(ahead ? kres_next : kres, voffK[j >> 1], step_off_k(tc), stage, wave, j >> 1);
+    if (j & 1)
+      R[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+          ahead ? qres_next : qres, (int)((unsigned)voffQ[j >> 1] + (unsigned)step_off_q(tc)), 0, 0));
+    else
+      R[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+          ahead ? kres_next : kres, (int)((unsigned)voffK[j >> 1] + (unsigned)step_off_k(tc)), 0, 0));
   };
-  // the workgroup's first tile: all of step 0 and the first two copies of step 1, then its first fragments
+  const int lane_dst = wave * 8 * 128 + lane * 16;
+  auto write_j = [&](int j, char* stage) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4*>(stage + (j & 1) * kTile * 128 + (j >> 1) * 64 * 128 + lane_dst) = R[j];
+  };
+  // Workgroup barrier that waits for this wavefront's LDS accesses only: the loads in flight into R must not be
+  // drained here (a __syncthreads() would wait for them).
+  auto lds_barrier = [&]() __attribute__((always_inline)) {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  };
+  // the workgroup's first tile: step 0 into stage 0, step 1 into the registers, then its first fragments
 #pragma unroll
-  for (int j = 0; j < 8; ++j) copy_j(j, 0, lds);
+  for (int j = 0; j < 8; ++j) load_j(j, 0);
 #pragma unroll
-  for (int j = 0; j < 2; ++j) copy_j(j, 1, lds + kStageBytes);
-  wait_vm0();
-  __syncthreads();
+  for (int j = 0; j < 8; ++j) write_j(j, lds);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) load_j(j, 1);
+  lds_barrier();
   bf16x8 fa[2][4], fb[2][2];
 #pragma unroll
   for (int x = 0; x < 4; ++x) fa[0][x] = read_frag(lds, wn * kSub + x * 32 + r, hh);
@@ -252,11 +269,10 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
 #pragma unroll
     for (int ss = 0; ss < 4; ++ss) {
       if (ss == 3) {
-        // every copy of step t+1 has landed; every wavefront has read its last
+        // every piece of step t+1 has been written to the other stage; every wavefront has read its last
         // fragment of step t (the reads were issued during sub-step 2)
         __builtin_amdgcn_sched_barrier(0);
-        wait_vm0();
-        __syncthreads();
+        lds_barrier();
       }
       const char* fragK = ss < 3 ? cur : nxt;             // where the next sub-step's fragments live
       const char* fragQ = fragK + kTile * 128;
@@ -264,9 +280,15 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         __builtin_amdgcn_sched_barrier(0);
+        {
+          // pieces 0..2 | 3..5 | 6..7 of step t+1 go to the other stage; their registers then take step t+2
+          const int j = ss * 3 + c;
+          if (ss < 3 && c < 3 && j < 8) {
+            write_j(j, nxt);
+            load_j(j, t + 2);
+          }
+        }
         if (c < 2) {
-          if (ss < 3) copy_j(2 + ss * 2 + c, t + 1, nxt);  // copies 2..7 of step t+1
-          else copy_j(c, t + 2, cur);                      // copies 0..1 of step t+2 refill this stage
           fa[(ss + 1) & 1][2 * c] = read_frag(fragK, wn * kSub + (2 * c) * 32 + r, nss * 2 + hh);
           fa[(ss + 1) & 1][2 * c + 1] = read_frag(fragK, wn * kSub + (2 * c + 1) * 32 + r, nss * 2 + hh);
         } else if (c == 2) {
@@ -387,7 +409,6 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   qres = qres_next;
   kres = kres_next;
   }   // tiles of this workgroup
-  wait_vm0();   // the repeats the last tile issued into LDS
 }
 
 // The arithmetic of the normalisation, shared by the stand-alone pass and the fused normalise-and-select kernel
