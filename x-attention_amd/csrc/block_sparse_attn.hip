@@ -192,15 +192,19 @@ __device__ __forceinline__ void pv_tile(const char* Vs, const int (&vaddr)[4][2]
   }
 }
 
-// token-level masking of one tile's scores: keys past the sequence end, and (causal) keys after the query
+// token-level masking of one tile's scores: keys past the sequence end, and (causal) keys after the query.
+// The lane's last visible key is taken relative to its first key of the tile once, so that each score costs one
+// compare against a constant and one select.
 __device__ __forceinline__ void mask_tile(f32x16 (&sacc)[4], int kb, int hh, int q_pos, int Lk, int causal) {
+  int last = Lk - 1;
+  if (causal) last = last < q_pos ? last : q_pos;
+  const int lim = last - kb * kBlk - hh * 4;
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int kpos = kb * kBlk + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
-      const bool dead = kpos >= Lk || (causal && kpos > q_pos);
-      sacc[nt][v] = dead ? -INFINITY : sacc[nt][v];
+      const int c = nt * 32 + (v >> 2) * 8 + (v & 3);     // key offset inside the tile, without the lane's hh * 4
+      sacc[nt][v] = c > lim ? -INFINITY : sacc[nt][v];
     }
 }
 
@@ -254,7 +258,7 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
 
   const int q_row = qb * kBlk + wave * 32 + r;          // this lane's query token
   const int q_pos = q_row + p.kv_off;                   // its position on the key axis
-  int n_blocks;
+  int n_blocks, first = 0;
   // the column list is read through the scalar cache (uniform, read-only), so that
   // fetching the next block id never waits on the tile copies in flight
   const_i32_ptr list = nullptr;
@@ -266,6 +270,7 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
       const int64_t slot = (int64_t)head * p.idx_rows + (qb - p.idx_row0);
       list = (const_i32_ptr)(uintptr_t)(p.col_idx + slot * p.idx_pitch);
       n_blocks = ((const_i32_ptr)(uintptr_t)p.col_cnt)[slot];
+      first = list[0];                     // idx_pitch >= 1: readable whatever the count
       n_blocks = n_blocks < 0 ? 0 : (n_blocks > p.idx_pitch ? (int)p.idx_pitch : n_blocks);
     } else {
       n_blocks = visible;
@@ -292,7 +297,7 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     tile_offsets(p.q_sn, lane, wave, voffQ);
     copy_tile(qbase, p.q_sn, p.Lq, qb, voffQ, Vs, wave);
     if (n_blocks > 0) {
-      kb = kHasList ? clamp_block(list[0], p.nkb) : 0;
+      kb = kHasList ? clamp_block(first, p.nkb) : 0;
       copy_tile(kbase, p.k_sn, p.Lk, kb, la.voffK, Ks, wave);
     }
     wait_vm0();
@@ -302,8 +307,9 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
     asm volatile("" ::: "memory");
     if (n_blocks > 0) copy_tile_async(vbase, p.v_sn, p.Lk, kb, la.voffV, Vs, wave);
   }
-  wait_vm0();
-  __syncthreads();                         // K_0 (and V_0) landed and visible
+  // K_0 landed before the fragments were read (every wavefront waited for its share); V_0 stays in flight during
+  // the first Q.K^T and is waited for with the tile's own barrier
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
   for (int j = 0; j < n_blocks; ++j) {
     const int kb_next = (j + 1 < n_blocks) ? (kHasList ? clamp_block(list[j + 1], p.nkb) : j + 1) : -1;
