@@ -230,9 +230,9 @@ def flops_and_bytes(w, L, chunk, n_sel):
     vis = 0.5 if causal else 1.0
     pass_bytes = 4.0 * H * n_r * nkb_p * vis + 2 * 4.0 * H * n_r * (n_r / 128.0) * vis + 4.0 * (n_sel + H * nkb_p)
     # the selection as the reference stages it: the full block-sum matrix in, a byte mask and the lists out
-    survey_bytes = H * nkb_p * nkb_p * 5 + 4.0 * (n_sel + H * nkb_p)
+    staging_bytes = H * nkb_p * nkb_p * 5 + 4.0 * (n_sel + H * nkb_p)
     return dict(full_blocks=full_blocks, f_est=f_est, f_dense=f_dense, f_sparse=f_sparse, pass_bytes=pass_bytes,
-                survey_bytes=survey_bytes, rbs=rbs)
+                staging_bytes=staging_bytes, rbs=rbs)
 
 
 def measure(w, q, k, v, L, tau, chunk, steps, warmup, dense_steps, dense_warmup):
@@ -327,7 +327,7 @@ def summarize(w, L, tau, chunk, m, headline_traffic=False):
         "kernel": "estimate_select_kernel (normalisation + selection, block sums in LDS)", "bound": "hbm",
         "achieved": round(sel_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(sel_gbs / PEAK_HBM_GBS, 4),
         "ms": round(t_sel, 3), "bytes": fb["pass_bytes"],
-        "reference_staging_bytes": fb["survey_bytes"],     # full block-sum matrix in, byte mask + lists out
+        "reference_staging_bytes": fb["staging_bytes"],     # full block-sum matrix in, byte mask + lists out
         "traffic": measured_traffic_bytes("xattn::estimate_select_kernel") if headline_traffic else None,
     }
     return {
