@@ -120,28 +120,45 @@ __device__ __forceinline__ bf16x8 read_frag(const char* slab, int row, int chunk
 // query tile row, which share their K' slabs across heads and their Q' slabs
 // across key tiles in that XCD's L2, and every XCD gets the same number of tiles.
 // Returns false when id is past the last tile.
-__device__ __forceinline__ bool decode_tile(const EstParams& p, int64_t id, int* head, int* m0, int* n0) {
-  const int64_t lin = ((id >> 8) * 8 + (id & 7)) * 32 + ((id >> 3) & 31);
-  if (lin >= p.total_tiles) return false;
-  const int G = p.H / p.Hkv;
-  const int per_group = p.tiles_per_head * G;
-  const int g = (int)(lin / per_group);
-  int rem = (int)(lin % per_group);
-  *head = g * G + rem % G;
-  int tt = rem / G;
-  int mt_row = 0, nt_first = 0;
-  for (;; ++mt_row) {
-    const int mfirst = p.row_begin + mt_row * kTile;
+//
+// A workgroup visits its tiles in increasing order, so the search for a tile's query-tile row resumes from the
+// row of the previous tile (TileCursor) instead of walking all rows again: between two tiles of a workgroup the
+// matrix pipes have nothing to do, and a walk over 32 rows with their visibility limits was 6 % of a tile's time.
+struct TileCursor {
+  int g = -1;          // KV group of the previous tile
+  int mt_row = 0;      // its query-tile row
+  int row_base = 0;    // (row, key tile) pairs of the group before that row
+};
+
+__device__ __forceinline__ bool decode_tile(const EstParams& p, int64_t id, TileCursor& c, int* head, int* m0, int* n0) {
+  const int64_t lin64 = ((id >> 8) * 8 + (id & 7)) * 32 + ((id >> 3) & 31);
+  if (lin64 >= p.total_tiles) return false;
+  const uint32_t lin = (uint32_t)lin64;                  // the host refuses launches of 2^31 tiles or more
+  const uint32_t G = (uint32_t)(p.H / p.Hkv);
+  const uint32_t per_group = (uint32_t)p.tiles_per_head * G;
+  const uint32_t g = lin / per_group;
+  const uint32_t rem = lin - g * per_group;
+  *head = (int)(g * G + rem % G);
+  const int tt = (int)(rem / G);                          // the tile among the group's (row, key tile) pairs
+  if ((int)g != c.g) {
+    c.g = (int)g;
+    c.mt_row = 0;
+    c.row_base = 0;
+  }
+  int nt_first = 0;
+  for (;;) {
+    const int mfirst = p.row_begin + c.mt_row * kTile;
     const int mlast = (mfirst + kTile - 1 < p.row_end ? mfirst + kTile - 1 : p.row_end - 1);
     int hi = row_hi(p, mlast) / kTile;
     hi = hi < p.nNT - 1 ? hi : p.nNT - 1;
     nt_first = row_lo(p, mfirst) / kTile;
     const int cnt = hi - nt_first + 1;
-    if (tt < cnt || mt_row + 1 >= p.nMT) break;
-    tt -= cnt;
+    if (tt < c.row_base + cnt || c.mt_row + 1 >= p.nMT) break;
+    c.row_base += cnt;
+    ++c.mt_row;
   }
-  *m0 = p.row_begin + mt_row * kTile;
-  *n0 = (nt_first + tt) * kTile;
+  *m0 = p.row_begin + c.mt_row * kTile;
+  *n0 = (nt_first + (tt - c.row_base)) * kTile;
   return true;
 }
 
@@ -161,7 +178,8 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   // first fragments, so after the epilogue (which needs no LDS) the next tile starts at full speed.
   int64_t id = blockIdx.x;
   int head, m0, n0;
-  if (!decode_tile(p, id, &head, &m0, &n0)) return;
+  TileCursor cursor;
+  if (!decode_tile(p, id, cursor, &head, &m0, &n0)) return;
 
   const int64_t q_snb = p.q_sn * 2, k_snb = p.k_sn * 2;
   const int64_t span = (int64_t)kTile * p.S;
@@ -250,7 +268,7 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   for (;;) {
   const int64_t id_next = id + gridDim.x;
   int head_next, m0_next, n0_next;
-  const bool more = decode_tile(p, id_next, &head_next, &m0_next, &n0_next);
+  const bool more = decode_tile(p, id_next, cursor, &head_next, &m0_next, &n0_next);
   if (more) {
     qres_next = q_resource(head_next, m0_next);
     kres_next = k_resource(head_next, n0_next);
@@ -309,6 +327,9 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   const int T = nbase / kSub;
   if (nbase < p.n_rk) {
   float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
+  const uint32_t row_bytes = (uint32_t)p.rows * 4u;      // one key block's row of P
+  // (the host keeps a head's share of P below 2 GiB, so byte offsets fit 31 bits)
+  const __amdgpu_buffer_rsrc_t pres = __builtin_amdgcn_make_buffer_rsrc((void*)Pst, 0, (int)((uint32_t)p.nkb * row_bytes), 0x00020000);
   float* Mst = p.Mt + ((int64_t)head * p.nT + T) * p.rows;
   float* Lst = p.Lt + ((int64_t)head * p.nT + T) * p.rows;
   // every key of this wavefront tile visible to every one of its query rows?
@@ -354,6 +375,13 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     float tot = 0.f;
     const int mrel = m - p.row_begin;
     constexpr int G = RBS / 8;   // 8-key groups (one per accumulator quad pair) per key block
+    // Partial sums leave through buffer stores with all 64 lanes active: the two half-waves hold the same sums
+    // after half_sum(), so half 0 stores one key block and half 1 the next one in the same instruction (its row
+    // of P lies `rows` floats further on); the key block's offset is uniform and travels in a scalar register.
+    // Lanes with nothing to store get an offset past the end of the buffer, which drops the store.
+    constexpr uint32_t kDropped = 0x80000000u;
+    const uint32_t lane_off = (uint32_t)mrel * 4u + (G < 4 ? (uint32_t)hh * row_bytes : 0u);
+    const int kb_first = nbase / RBS;      // first key block of this wavefront tile (uniform)
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       float part[4];
@@ -376,20 +404,22 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
       // part[g] covers keys nbase + nt*32 + 8g .. +7
       if (G == 1) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int kb = (nbase + nt * 32 + g * 8) / RBS;
-          if (row_ok && kb < p.nkb && hh == (g & 1)) Pst[(int64_t)kb * p.rows + mrel] = part[g];
+        for (int q2 = 0; q2 < 2; ++q2) {       // key blocks kb, kb + 1 by half-wave 0, 1
+          const int kb = kb_first + nt * 4 + q2 * 2;
+          const float val = hh ? part[2 * q2 + 1] : part[2 * q2];
+          const uint32_t off = (row_ok && kb + hh < p.nkb) ? lane_off : kDropped;
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), pres, (int)off, (int)((uint32_t)kb * row_bytes), 0);
         }
       } else if (G == 2) {
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          const int kb = (nbase + nt * 32 + g * 16) / RBS;
-          if (row_ok && kb < p.nkb && hh == g) Pst[(int64_t)kb * p.rows + mrel] = part[2 * g] + part[2 * g + 1];
-        }
+        const int kb = kb_first + nt * 2;
+        const float val = hh ? part[2] + part[3] : part[0] + part[1];
+        const uint32_t off = (row_ok && kb + hh < p.nkb) ? lane_off : kDropped;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), pres, (int)off, (int)((uint32_t)kb * row_bytes), 0);
       } else {
-        const int kb = (nbase + nt * 32) / RBS;
-        if (row_ok && kb < p.nkb && hh == 0)
-          Pst[(int64_t)kb * p.rows + mrel] = part[0] + part[1] + part[2] + part[3];
+        const int kb = kb_first + nt;
+        const float val = part[0] + part[1] + part[2] + part[3];
+        const uint32_t off = (row_ok && kb < p.nkb && hh == 0) ? lane_off : kDropped;
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), pres, (int)off, (int)((uint32_t)kb * row_bytes), 0);
       }
     }
     if (row_ok && hh == 0) {
@@ -867,6 +897,8 @@ int estimate_impl(const void* q, const void* k, float* block_sums, void* workspa
     p.win_rows = window_rows;
   }
   if (workspace_size < workspace_bytes(num_heads, g, p.rows)) return XATTN_ERR_WORKSPACE;
+  // the kernel addresses one head's partial sums with 31-bit byte offsets
+  if ((int64_t)g.nkb * p.rows * 4 >= 0x7fffffff) return XATTN_ERR_SHAPE;
   float* ws = static_cast<float*>(workspace);
   p.P = ws;
   p.Mt = ws + (size_t)num_heads * g.nkb * p.rows;
