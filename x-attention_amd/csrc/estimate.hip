@@ -327,9 +327,6 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
   const int T = nbase / kSub;
   if (nbase < p.n_rk) {
   float* Pst = p.P + (int64_t)head * p.nkb * p.rows;
-  const uint32_t row_bytes = (uint32_t)p.rows * 4u;      // one key block's row of P
-  // (the host keeps a head's share of P below 2 GiB, so byte offsets fit 31 bits)
-  const __amdgpu_buffer_rsrc_t pres = __builtin_amdgcn_make_buffer_rsrc((void*)Pst, 0, (int)((uint32_t)p.nkb * row_bytes), 0x00020000);
   float* Mst = p.Mt + ((int64_t)head * p.nT + T) * p.rows;
   float* Lst = p.Lt + ((int64_t)head * p.nT + T) * p.rows;
   // every key of this wavefront tile visible to every one of its query rows?
@@ -375,13 +372,6 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
     float tot = 0.f;
     const int mrel = m - p.row_begin;
     constexpr int G = RBS / 8;   // 8-key groups (one per accumulator quad pair) per key block
-    // Partial sums leave through buffer stores with all 64 lanes active: the two half-waves hold the same sums
-    // after half_sum(), so half 0 stores one key block and half 1 the next one in the same instruction (its row
-    // of P lies `rows` floats further on); the key block's offset is uniform and travels in a scalar register.
-    // Lanes with nothing to store get an offset past the end of the buffer, which drops the store.
-    constexpr uint32_t kDropped = 0x80000000u;
-    const uint32_t lane_off = (uint32_t)mrel * 4u + (G < 4 ? (uint32_t)hh * row_bytes : 0u);
-    const int kb_first = nbase / RBS;      // first key block of this wavefront tile (uniform)
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       float part[4];
@@ -404,22 +394,20 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
       // part[g] covers keys nbase + nt*32 + 8g .. +7
       if (G == 1) {
 #pragma unroll
-        for (int q2 = 0; q2 < 2; ++q2) {       // key blocks kb, kb + 1 by half-wave 0, 1
-          const int kb = kb_first + nt * 4 + q2 * 2;
-          const float val = hh ? part[2 * q2 + 1] : part[2 * q2];
-          const uint32_t off = (row_ok && kb + hh < p.nkb) ? lane_off : kDropped;
-          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), pres, (int)off, (int)((uint32_t)kb * row_bytes), 0);
+        for (int g = 0; g < 4; ++g) {
+          const int kb = (nbase + nt * 32 + g * 8) / RBS;
+          if (row_ok && kb < p.nkb && hh == (g & 1)) Pst[(int64_t)kb * p.rows + mrel] = part[g];
         }
       } else if (G == 2) {
-        const int kb = kb_first + nt * 2;
-        const float val = hh ? part[2] + part[3] : part[0] + part[1];
-        const uint32_t off = (row_ok && kb + hh < p.nkb) ? lane_off : kDropped;
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), pres, (int)off, (int)((uint32_t)kb * row_bytes), 0);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          const int kb = (nbase + nt * 32 + g * 16) / RBS;
+          if (row_ok && kb < p.nkb && hh == g) Pst[(int64_t)kb * p.rows + mrel] = part[2 * g] + part[2 * g + 1];
+        }
       } else {
-        const int kb = kb_first + nt;
-        const float val = part[0] + part[1] + part[2] + part[3];
-        const uint32_t off = (row_ok && kb < p.nkb && hh == 0) ? lane_off : kDropped;
-        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), pres, (int)off, (int)((uint32_t)kb * row_bytes), 0);
+        const int kb = (nbase + nt * 32) / RBS;
+        if (row_ok && kb < p.nkb && hh == 0)
+          Pst[(int64_t)kb * p.rows + mrel] = part[0] + part[1] + part[2] + part[3];
       }
     }
     if (row_ok && hh == 0) {
@@ -897,8 +885,6 @@ int estimate_impl(const void* q, const void* k, float* block_sums, void* workspa
     p.win_rows = window_rows;
   }
   if (workspace_size < workspace_bytes(num_heads, g, p.rows)) return XATTN_ERR_WORKSPACE;
-  // the kernel addresses one head's partial sums with 31-bit byte offsets
-  if ((int64_t)g.nkb * p.rows * 4 >= 0x7fffffff) return XATTN_ERR_SHAPE;
   float* ws = static_cast<float*>(workspace);
   p.P = ws;
   p.Mt = ws + (size_t)num_heads * g.nkb * p.rows;
