@@ -349,67 +349,75 @@ __global__ __launch_bounds__(512) void estimate_gemm_kernel(EstParams p) {
           if (n < p.n_rk) dst[n] = acc[nt][mt][v];
         }
     }
-    // pass 1: row maximum over this tile's visible keys (exp2 domain)
-    float mx = -INFINITY;
-    if (all_visible) {
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc[nt][mt][v]);
-      mx *= p.scale_log2;   // scale > 0
-    } else {
+    // Tiles on the diagonal or at the sequence end first overwrite the scores of invisible keys with -inf: they
+    // then drop out of the maximum and exponentiate to zero, and the two passes below need neither a test per
+    // score nor a second copy.
+    if (!all_visible) {
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int n = nbase + nt * 32 + (v >> 2) * 8 + hh * 4 + (v & 3);
           const bool vis = n >= lo && n <= hi && n < p.n_rk;
-          mx = fmaxf(mx, vis ? acc[nt][mt][v] * p.scale_log2 : -INFINITY);
+          acc[nt][mt][v] = vis ? acc[nt][mt][v] : -INFINITY;
         }
     }
+    // pass 1: row maximum over this tile's visible keys (exp2 domain)
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc[nt][mt][v]);
+    mx *= p.scale_log2;   // scale > 0
     mx = half_max(mx);
     const float safe = (mx == -INFINITY) ? 0.f : mx;
     float tot = 0.f;
     const int mrel = m - p.row_begin;
     constexpr int G = RBS / 8;   // 8-key groups (one per accumulator quad pair) per key block
+    // what the stores below share: the first key block of this wavefront tile and how many of its key blocks
+    // exist (uniform), the row of P they start from (uniform) and each half-wave's predicate
+    const int kb_first = (int)((uint32_t)nbase / (uint32_t)RBS);
+    const int kb_left = p.nkb - kb_first;
+    float* const prow = Pst + (int64_t)kb_first * p.rows + mrel;
+    const int64_t rows64 = p.rows;
+    const bool st0 = row_ok && hh == 0, st1 = row_ok && hh == 1;
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
-      float part[4];
+      float s[4];       // this lane's share of the sums over keys nbase + nt*32 + 8g .. +7 (the other half-wave has the rest)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        float s = 0.f;
+        s[g] = 0.f;
 #pragma unroll
         for (int t2 = 0; t2 < 4; ++t2) {
           const int v = g * 4 + t2;
-          float e = fast_exp2(__builtin_fmaf(acc[nt][mt][v], p.scale_log2, -safe));
-          if (!all_visible) {
-            const int n = nbase + nt * 32 + g * 8 + hh * 4 + t2;
-            e = (n >= lo && n <= hi && n < p.n_rk) ? e : 0.f;
-          }
-          s += e;
+          s[g] += fast_exp2(__builtin_fmaf(acc[nt][mt][v], p.scale_log2, -safe));
         }
-        part[g] = half_sum(s);
-        tot += part[g];
       }
-      // part[g] covers keys nbase + nt*32 + 8g .. +7
+      // Key blocks go out in pairs: one swap leaves the first block's sum in the lower half-wave and the second
+      // block's in the upper one, which are the lanes that store them.  tot adds up what a lane stores; the two
+      // half-waves are combined once at the end.
       if (G == 1) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int kb = (nbase + nt * 32 + g * 8) / RBS;
-          if (row_ok && kb < p.nkb && hh == (g & 1)) Pst[(int64_t)kb * p.rows + mrel] = part[g];
+        for (int q2 = 0; q2 < 2; ++q2) {
+          const float both = half_sum_pair(s[2 * q2], s[2 * q2 + 1]);
+          tot += both;
+          const int k = nt * 4 + 2 * q2;
+          if (k < kb_left && st0) prow[k * rows64] = both;
+          if (k + 1 < kb_left && st1) prow[(k + 1) * rows64] = both;
         }
       } else if (G == 2) {
-#pragma unroll
-        for (int g = 0; g < 2; ++g) {
-          const int kb = (nbase + nt * 32 + g * 16) / RBS;
-          if (row_ok && kb < p.nkb && hh == g) Pst[(int64_t)kb * p.rows + mrel] = part[2 * g] + part[2 * g + 1];
-        }
+        const float both = half_sum_pair(s[0] + s[1], s[2] + s[3]);
+        tot += both;
+        const int k = nt * 2;
+        if (k < kb_left && st0) prow[k * rows64] = both;
+        if (k + 1 < kb_left && st1) prow[(k + 1) * rows64] = both;
       } else {
-        const int kb = (nbase + nt * 32) / RBS;
-        if (row_ok && kb < p.nkb && hh == 0)
-          Pst[(int64_t)kb * p.rows + mrel] = part[0] + part[1] + part[2] + part[3];
+        const float all = half_sum(s[0] + s[1] + s[2] + s[3]);
+        tot += hh == 0 ? all : 0.f;
+        if (nt < kb_left && st0) prow[nt * rows64] = all;
       }
     }
+    tot = half_sum(tot);
     if (row_ok && hh == 0) {
       Mst[mrel] = mx;
       Lst[mrel] = tot;

@@ -53,6 +53,12 @@ __device__ __forceinline__ void half_pair(float x, float& lo, float& hi) {
   hi = x;
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
 }
+// Two values combined across the half-waves at once: the lower half-wave ends up with a of the lane plus a of its
+// partner, the upper half-wave with b plus b of its partner - one swap where two half_sum() calls need two.
+__device__ __forceinline__ float half_sum_pair(float a, float b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
 __device__ __forceinline__ float half_sum(float x) {
   float lo, hi;
   half_pair(x, lo, hi);
