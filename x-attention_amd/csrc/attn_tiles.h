@@ -98,20 +98,35 @@ __host__ __device__ inline DispatchShape dispatch_shape(int H, int Hkv) {
   return d;
 }
 
-// Returns false for ids that carry no work.
-__host__ __device__ inline bool map_workgroup(int id, int H, int Hkv, int qb_begin, int qb_end, int* head, int* qb) {
+// Returns false for ids that carry no work.  The shape is computed once on the host (dispatch_shape) and the
+// arithmetic is unsigned: this runs at the start of every workgroup, where its divisions are a measurable part
+// of what a short unit costs.
+__host__ __device__ inline bool map_workgroup(int id, const DispatchShape& d, int qb_begin, int qb_end, int* head,
+                                              int* qb, int* kv_head) {
   if (id < 0) return false;
-  const DispatchShape d = dispatch_shape(H, Hkv);
-  const int x = id & 7, s = id >> 3;
-  const int unit = (s / kUnit) * 8 + x, w = s % kUnit;
-  const int run = unit / d.n_groups;
-  const int dg = (unit % d.n_groups + run) % d.n_groups;
-  const int from_end = run * d.unit_rows + w / d.set_heads;
-  const int in_group = (dg % d.sets) * d.set_heads + w % d.set_heads;   // head index inside its KV group
-  if (w >= d.set_heads * d.unit_rows || from_end >= qb_end - qb_begin || in_group >= d.group) return false;
-  *qb = qb_end - 1 - from_end;
-  *head = (dg / d.sets) * d.group + in_group;
+  const uint32_t x = (uint32_t)id & 7u, s = (uint32_t)id >> 3;
+  const uint32_t unit = (s / kUnit) * 8u + x, w = s % kUnit;
+  const uint32_t ng = (uint32_t)d.n_groups, sh = (uint32_t)d.set_heads;
+  const uint32_t run = unit / ng;
+  const uint32_t dg = (unit + run) % ng;      // the unit's group, rotated by its run
+  const uint32_t w_row = w / sh, w_head = w - w_row * sh;
+  const uint32_t from_end = run * (uint32_t)d.unit_rows + w_row;
+  uint32_t set = 0, kvh = dg;
+  if (d.sets != 1) {
+    kvh = dg / (uint32_t)d.sets;
+    set = dg - kvh * (uint32_t)d.sets;
+  }
+  const uint32_t in_group = set * sh + w_head;             // head index inside its KV group
+  if (w >= sh * (uint32_t)d.unit_rows || from_end >= (uint32_t)(qb_end - qb_begin) || in_group >= (uint32_t)d.group)
+    return false;
+  *qb = qb_end - 1 - (int)from_end;
+  *head = (int)(kvh * (uint32_t)d.group + in_group);
+  *kv_head = (int)kvh;
   return true;
+}
+__host__ __device__ inline bool map_workgroup(int id, int H, int Hkv, int qb_begin, int qb_end, int* head, int* qb) {
+  int kv_head;
+  return map_workgroup(id, dispatch_shape(H, Hkv), qb_begin, qb_end, head, qb, &kv_head);
 }
 
 // grid size of a launch over n_qblocks q-blocks

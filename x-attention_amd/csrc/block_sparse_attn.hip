@@ -48,6 +48,7 @@ struct AttnParams {
   int qb_begin, qb_end;     // q-blocks handled by this launch
   int causal, kv_off;       // kv_off = Lk - Lq
   float scale_log2;         // softmax_scale * log2(e)
+  DispatchShape shape;      // dispatch_shape(H, Hkv), computed on the host
 };
 
 __device__ __forceinline__ int clamp_block(int kb, int nkb) { return kb < 0 ? 0 : (kb < nkb ? kb : nkb - 1); }
@@ -227,14 +228,21 @@ __device__ __forceinline__ void store_out(const AttnParams& p, int head, int qb,
       const int c = dt * 4 + g;                          // 16-byte chunk of the row; XOR-swizzled against bank conflicts
       *reinterpret_cast<u32x2*>(stage + r * 256 + ((c ^ (r & 15)) << 4) + hh * 8) = w;
     }
-  // written and read by the same wavefront: the LDS keeps a wavefront's accesses in order, no barrier
+  // written and read by the same wavefront: the LDS keeps a wavefront's accesses in order, no barrier.
+  // The rows leave through a buffer resource that ends with the sequence (rows past it are dropped), rebased to
+  // the q-block so that a lane's offset is one 32-bit product plus a multiple of four rows.
+  const int rows_left = p.Lq - qb * kBlk;
+  const int rows = rows_left < kBlk ? rows_left : kBlk;
+  const __amdgpu_buffer_rsrc_t ores = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)(p.o + (int64_t)head * p.o_sh + (int64_t)qb * kBlk * p.o_sn), 0, (int)((int64_t)rows * p.o_sn * 2), 0x00020000);
   const int c = lane & 15;
+  const uint32_t row_bytes = (uint32_t)p.o_sn * 2u;
+  const uint32_t voff0 = (uint32_t)(wave * 32 + (lane >> 4)) * row_bytes + (uint32_t)c * 16u;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int row = i * 4 + (lane >> 4);
     const u32x4 w = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c ^ (row & 15)) << 4));
-    const int q_row = qb * kBlk + wave * 32 + row;
-    if (q_row < p.Lq) *reinterpret_cast<u32x4*>(p.o + (int64_t)head * p.o_sh + (int64_t)q_row * p.o_sn + c * 8) = w;
+    __builtin_amdgcn_raw_buffer_store_b128(w, ores, (int)(voff0 + (uint32_t)(i * 4) * row_bytes), 0, 0);
   }
 }
 
@@ -249,9 +257,8 @@ __global__ __launch_bounds__(256, 2) void block_sparse_fwd_kernel(AttnParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hh = lane >> 5;
 
-  int head, qb;
-  if (!map_workgroup(blockIdx.x, p.H, p.Hkv, p.qb_begin, p.qb_end, &head, &qb)) return;
-  const int kvh = head / (p.H / p.Hkv);
+  int head, qb, kvh;
+  if (!map_workgroup(blockIdx.x, p.shape, p.qb_begin, p.qb_end, &head, &qb, &kvh)) return;
   const __bf16* qbase = p.q + (int64_t)head * p.q_sh;
   const __bf16* kbase = p.k + (int64_t)kvh * p.k_sh;
   const __bf16* vbase = p.v + (int64_t)kvh * p.v_sh;
@@ -357,7 +364,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   for (int64_t s : strides)
     if (s % 8) return XATTN_ERR_ALIGN;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return XATTN_ERR_ALIGN;
-  if (!tile_stride_ok(k_stride_n) || !tile_stride_ok(v_stride_n) || !tile_stride_ok(q_stride_n) || o_stride_n < kHeadDim)
+  if (!tile_stride_ok(k_stride_n) || !tile_stride_ok(v_stride_n) || !tile_stride_ok(q_stride_n) || !tile_stride_ok(o_stride_n))
     return XATTN_ERR_SHAPE;
   if (!scale_ok(softmax_scale)) return XATTN_ERR_SHAPE;
 
@@ -384,6 +391,7 @@ extern "C" int xattn_block_sparse_fwd(const void* q, const void* k, const void* 
   p.idx_row0 = idx_row0;
   p.qb_begin = q_block_begin;
   p.qb_end = q_block_end;
+  p.shape = dispatch_shape(p.H, p.Hkv);
   const int64_t grid = grid_for(p.H, p.Hkv, q_block_end - q_block_begin);
   if (grid > 0x7fffffff) return XATTN_ERR_SHAPE;
   if (col_idx)
