@@ -205,8 +205,8 @@ int xattn_estimate_select(const void* q, const void* k, float* block_sums, void*
  * the baseline the speedup is quoted against.  Only query blocks
  * [q_block_begin, q_block_end) are computed (q_block_end < 0: up to the last),
  * so query chunks can be launched as their block lists become available.
- * Token strides of q, k and v: 128 .. 2^22 elements (all three are moved as
- * 128-row tiles whose byte offsets are held in 32 bits); of out: >= 128.
+ * Token strides of q, k, v and out: 128 .. 2^22 elements (all four are moved
+ * as 128-row tiles whose byte offsets are held in 32 bits).
  */
 int xattn_block_sparse_fwd(const void* q, const void* k, const void* v, void* out,
                            const int32_t* col_idx, const int32_t* col_cnt, int64_t idx_pitch,
